@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SWM_ABI_VERSION 2
+#define SWM_ABI_VERSION 3
 int swm_abi_version(void);
 const char* swm_last_error(void);
 
@@ -157,15 +157,16 @@ int swm_clamped_glu(void* out, const void* in, int64_t in_stride, int64_t rows, 
 /* out[rows, ff] = max(in, 0)^2 */
 int swm_relu2(void* out, const void* in, int64_t in_stride, int64_t rows, int ff, int act_dtype, void* stream);
 
-/* Rotary embedding on neighbouring pairs (2i, 2i + 1) of the first rot_dims coordinates of every head, angle
+/* Rotary embedding on the first rot_dims coordinates of every head: pair i is the neighbours (2i, 2i + 1), or with
+ * pair_halves != 0 the coordinates (i, i + rot_dims / 2); angle
  * = float(positions[t]) * inv_freq[i] in fp32 (inv_freq fp32 [rot_dims / 2]); the other coordinates pass.
  * q_out fp32 [rows, heads * dim] = rotated q.  With k != NULL: key_cache[slot] = rotated k, value_cache[slot] = v
  * (slot = slot_mapping[t], < 0: not cached; caches [slots, kv_heads * dim | vdim] act_dtype).  q, k, v are column
  * ranges of one projection output (row stride in_stride). */
 int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, int64_t in_stride,
-                   const int64_t* positions, const float* inv_freq, int rot_dims, void* key_cache, void* value_cache,
-                   const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim, int vdim, int act_dtype,
-                   void* stream);
+                   const int64_t* positions, const float* inv_freq, int rot_dims, int pair_halves, void* key_cache,
+                   void* value_cache, const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim,
+                   int vdim, int act_dtype, void* stream);
 
 /* The choice of a mixture-of-experts router from its logits (fp32 [rows, experts], the router's product with the
  * layer input): s = sigmoid(logit); choice scores s + correction (NULL: none); experts form `groups` equal groups
@@ -192,6 +193,65 @@ int swm_capped_attention(void* out, const float* q, const void* key_cache, const
                          const int32_t* q_start, const int32_t* ctx_len, int64_t rows, int num_seqs,
                          int max_query_len, int heads, int kv_heads, int dim, int vdim, int page_size, float scale,
                          float softcap, int window, int act_dtype, void* stream);
+
+/* The same attention with the mask and the cache layout named: `window` > 0: position i sees j with 0 <= i - j <
+ * window; `chunk` > 0: i sees j <= i with j / chunk == i / chunk (chunks count from position 0 of the sequence); both
+ * 0: every j <= i.  `sink` != 0: the softmax's denominator has one more term, exp(0) (a key of score 0 without a
+ * value).  A cache slot (one token) holds k_stride / v_stride elements, of which key/value head g's begin at g * dim /
+ * g * vdim: value_cache may point into the key cache (values that are a part of the key row).  Key and value sizes up
+ * to 384. */
+int swm_masked_attention(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
+                         int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
+                         const int32_t* ctx_len, int64_t rows, int num_seqs, int max_query_len, int heads,
+                         int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
+                         int chunk, int sink, int64_t k_stride, int64_t v_stride, int act_dtype, void* stream);
+
+/* ---- layers whose sublayer outputs enter an fp32 stream through a gate, with a mix over all earlier layers ---- */
+
+/* v = stream[t] + mult * y[t] * sigmoid(gate[t])   (y NULL: v = stream[t]; gate NULL: no gate; y, gate act_dtype
+ * with row strides).  With `history` (fp32 [entries or more, rows, width], layer_stride floats apart): entry
+ * entries - 1 receives v, and v becomes sum_j depth_weights[j] * history[j] over the `entries` entries (fp32 weights).
+ * stream[t] = v.  With `out`: out[t] = act_dtype(tanh(norm_alpha[0] * v) * norm_weight + norm_bias), all fp32. */
+int swm_gated_stream_step(float* stream, const void* y, int64_t y_stride, const void* gate, int64_t gate_stride,
+                          float mult, float* history, int64_t layer_stride, const float* depth_weights, int entries,
+                          const float* norm_alpha, const float* norm_weight, const float* norm_bias, void* out,
+                          int64_t rows, int width, int act_dtype, void* stream_handle);
+
+/* out[t] = c0 U(z) + c1 U(z^2) + c2 U(z^3) + c3, powers element by element, U(u) = u / sqrt(mean(u^2) + eps) over the
+ * row's ff values; coef fp32 [4]; z act_dtype with row stride; out act_dtype [rows, ff]. */
+int swm_poly_norm(void* out, const void* z, int64_t z_stride, const float* coef, float eps, int64_t rows, int ff,
+                  int act_dtype, void* stream);
+
+/* out[t, h * size + c] = y[t, h, c] * sigmoid(gate[t, h * size + c])   (silu != 0: * gate * sigmoid(gate));
+ * y addressed as t * y_row_stride + h * y_head_stride + c. */
+int swm_gate_mul(void* out, const void* y, int64_t y_row_stride, int64_t y_head_stride, const void* gate,
+                 int64_t gate_stride, int64_t rows, int heads, int size, int silu, int act_dtype, void* stream);
+
+/* Attention over a low-rank latent: a token's cache row is its latent (rank) | one rotated key part (rot) shared by
+ * all heads.  cache[slot] = down[t, :rank] / sqrt(mean(.^2) + eps) * norm_weight | rotate(down[t, rank:rank + rot])
+ * (down NULL: no cache write); q_out[t, h] (fp32 [rows, heads * (rank + rot)]) = q_latent[t, h] | rotate(q_rot[t, h]),
+ * q_latent being the head's query already taken through the key up-projection.  Rotation on neighbouring pairs,
+ * angle = float(position) * inv_freq[i] (fp32 [rot / 2]).  q_latent, q_rot are addressed by row and head strides. */
+int swm_latent_rope_cache(float* q_out, const void* q_latent, int64_t ql_row_stride, int64_t ql_head_stride,
+                          const void* q_rot, int64_t qr_row_stride, int64_t qr_head_stride, const void* down,
+                          int64_t down_stride, const float* norm_weight, float eps, const int64_t* positions,
+                          const float* inv_freq, void* cache, const int64_t* slot_mapping, int64_t rows, int heads,
+                          int rank, int rot, int act_dtype, void* stream);
+
+/* The per-head output norm with the gate's activation named: gate_silu != 0 multiplies by gate * sigmoid(gate). */
+int swm_head_norm_gate_act(void* out, const float* o, const void* gate, int64_t gate_stride, const float* weight,
+                           int weight_head_stride, float eps, int64_t rows, int heads, int vdim, int gate_silu,
+                           int act_dtype, void* stream);
+
+/* Gated linear attention with a decay per head and key channel:  S <- diag(a_t) S + k_t v_t^T;  o_t = S^T q_t * q_scale,
+ * a_t = sigmoid(decay_pre + decay_bias)^(1 / tau), i.e. log a_t = logsigmoid(.) / tau, worked out in fp32.
+ * q, k [rows, heads * dim], v [rows, heads * vdim]: act_dtype column ranges of one projection output (row stride
+ * in_stride); decay_pre act_dtype [rows, heads * dim] (row stride decay_stride); decay_bias fp32 [heads * dim] (NULL:
+ * none); state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim].  Key size up to 256. */
+int swm_gla(float* out, const void* q, const void* k, const void* v, int64_t in_stride, const void* decay_pre,
+            int64_t decay_stride, const float* decay_bias, float tau, float q_scale, float* state,
+            const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows, int num_seqs,
+            int max_query_len, int heads, int dim, int vdim, int act_dtype, void* stream);
 
 /* Linear attention with one decay per head:  S <- decay[h] S + k v^T;  o = S^T q, with q, k, v = silu of the given
  * projections (act_dtype, column ranges of one output with row stride in_stride; q, k [rows, heads * dim],

@@ -1,5 +1,8 @@
 // Causal softmax attention of a ragged step over paged keys with grouped query heads, an optional soft cap on the
-// scores (cap * tanh(score / cap)), an optional sliding window and an optional sigmoid gate on the output.
+// scores (cap * tanh(score / cap)), an optional mask (a sliding window, or chunks counted from position 0 inside which
+// a position sees the earlier ones), an optional extra term exp(0) in the softmax's denominator (a key of score 0
+// that carries no value) and an optional sigmoid gate on the output.  A cache slot's keys and values are addressed
+// by strides, so values may be a part of the key rows (attention over a latent shared by all heads).
 // Scores, softmax weights and the weighted sum of values are fp32: both products run on the matrix cores in
 // fp32 (v_mfma_f32_32x32x2_f32), keys and values are widened when they come from a bf16 cache.
 //
@@ -24,6 +27,7 @@ namespace swm {
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 
 constexpr int kQT = 32;               // query rows and keys per tile
+constexpr int kMaxBlocks = 12;        // 32-coordinate blocks of the larger of key and value size
 
 // N consecutive elements of a cache row as they are stored (bf16 two to a register), widened where they are used:
 // all loads of a key tile are issued before its first product, so their latencies overlap.
@@ -107,7 +111,8 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     const void* __restrict__ value_cache, const void* __restrict__ gate, int64_t gate_stride,
     const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
-    float scale, float softcap, int window, int tpt, int split, int rows_used, int page_shift) {
+    float scale, float softcap, int window, int chunk, int sink, int64_t k_stride, int64_t v_stride, int tpt, int split,
+    int rows_used, int page_shift) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int R = heads / kv_heads;
   const int dblocks = (dim + 31) / 32;
@@ -147,9 +152,11 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
   // rows without a token behave like the tile's last token and are never stored
   const int pos_q = first_pos + min(qi / R, max(ntok - 1, 0));
   // keys below every row's window are skipped as whole tiles
-  const int lowest = window > 0 ? max(0, first_pos - window + 1) : 0;
+  const int lowest = chunk > 0 ? first_pos / chunk * chunk : window > 0 ? max(0, first_pos - window + 1) : 0;
+  // the first key that this lane's query sees: its chunk's first position, or the window's
+  const int low_q = chunk > 0 ? pos_q / chunk * chunk : window > 0 ? pos_q - window + 1 : 0;
   const int tile_lo = lowest / kQT, tile_hi = live ? last_pos / kQT : -1;
-  const bool kvec = dim % 8 == 0;
+  const bool kvec = dim % 8 == 0 && k_stride % 8 == 0;
   const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
 
   f32x16 o[NVB];
@@ -159,7 +166,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     for (int r = 0; r < 16; ++r) o[b][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
 
-  const bool vvec = is_pow2(NB) && vdim % NB == 0;
+  const bool vvec = is_pow2(NB) && vdim % NB == 0 && v_stride % NB == 0;
   const int kstep = split ? nw : 1;
   // cache slot of key k0 + qi of a tile (-1: beyond the tile's last key)
   auto slot_of = [&](int k0) {
@@ -170,7 +177,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
   };
   // loads of one key tile: this lane's key row (runs of 16 per block); the values of keys (r, hl)
   auto issue_keys = [&](int slot, Raw<T, 16> (&kraw)[NB]) {
-    const int64_t krow = ((int64_t)max(slot, 0) * kv_heads + g) * dim;
+    const int64_t krow = (int64_t)max(slot, 0) * k_stride + (int64_t)g * dim;
 #pragma unroll
     for (int b = 0; b < NB; ++b)
       if (b < dblocks) load_raw(kraw[b], key_cache, krow, b * 32 + hl * 16, dim, slot >= 0, kvec);
@@ -179,7 +186,8 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int vslot = __shfl(slot, 8 * (r / 4) + 4 * hl + (r % 4), 64);
-      load_raw(vraw[r], value_cache, ((int64_t)max(vslot, 0) * kv_heads + g) * vdim, qi * NB, vdim, vslot >= 0, vvec);
+      load_raw(vraw[r], value_cache, (int64_t)max(vslot, 0) * v_stride + (int64_t)g * vdim, qi * NB, vdim, vslot >= 0,
+               vvec);
     }
   };
   // A tile's values are asked for before its first product and arrive while it runs.  With a 16-bit cache and heads of
@@ -227,7 +235,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
       const int kj = k0 + 8 * (r / 4) + 4 * hl + (r % 4);
       float v = s[r];
       if (softcap > 0.0f) v = softcap * fast_tanhf_(v * inv_cap);
-      const bool seen = kj <= pos_q && (window <= 0 || pos_q - kj < window);
+      const bool seen = kj <= pos_q && kj >= low_q;
       v = seen ? v : -INFINITY;
       p[r] = v;
       tmax = fmaxf(tmax, v);
@@ -286,7 +294,8 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
       if (tt >= ntok) continue;
       float m_all = -INFINITY;
       for (int w = 0; w < nw; ++w) m_all = fmaxf(m_all, Ml[(w * kQT + r) * 2]);
-      float num = 0.0f, den = 0.0f;
+      if (sink) m_all = fmaxf(m_all, 0.0f);                  // one more term of score 0 that carries no value
+      float num = 0.0f, den = sink ? expf(-m_all) : 0.0f;
       for (int w = 0; w < nw; ++w) {
         const float f = expf(Ml[(w * kQT + r) * 2] - m_all);  // a wave that saw no key: exp(-inf) = 0
         den += f * Ml[(w * kQT + r) * 2 + 1];
@@ -302,7 +311,9 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
   // ---- every wave for itself: turn O^T round through the wave's own LDS region (its queries are done with)
   __syncthreads();
   if (live) {
-    const float inv = 1.0f / l_run;
+    const float m_fin = sink ? fmaxf(m_run, 0.0f) : m_run;
+    const float fin = sink ? expf(m_run - m_fin) : 1.0f;
+    const float inv = fin / (l_run * fin + (sink ? expf(-m_fin) : 0.0f));
 #pragma unroll
     for (int b = 0; b < NVB; ++b)
 #pragma unroll
@@ -332,7 +343,7 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
     const void* __restrict__ value_cache, const void* __restrict__ gate, int64_t gate_stride,
     const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, int heads, int kv_heads, int dim, int vdim, int page_size, int page_shift,
-    float scale, float softcap, int window) {
+    float scale, float softcap, int window, int chunk, int sink, int64_t k_stride, int64_t v_stride) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int seq = blockIdx.x, g = blockIdx.y, R = heads / kv_heads;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, pt = lane % LK, grp = lane / LK, nw = blockDim.x >> 6;
@@ -344,11 +355,12 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
   float* Os = lds + nw * RQ * 2;                             // [nw][RQ][LK * C]
 
   float qv[RQ][C], o[RQ][C], m_run[RQ], l_run[RQ];
-  int pos[RQ];
+  int pos[RQ], low[RQ];
 #pragma unroll
   for (int r = 0; r < RQ; ++r) {
     const int tt = r / R, hh = r % R;
     pos[r] = ctx + min(tt, n - 1);                           // padding rows behave like the last token's
+    low[r] = chunk > 0 ? pos[r] / chunk * chunk : window > 0 ? pos[r] - window + 1 : 0;
     m_run[r] = -INFINITY;
     l_run[r] = 0.0f;
 #pragma unroll
@@ -359,9 +371,10 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
       o[r][c] = 0.0f;
     }
   }
-  const bool kvec = dim % (C >= 8 ? 8 : 4) == 0, vvec = vdim % (C >= 8 ? 8 : 4) == 0;
+  constexpr int kPiece = C >= 8 ? 8 : 4;
+  const bool kvec = dim % kPiece == 0 && k_stride % kPiece == 0, vvec = vdim % kPiece == 0 && v_stride % kPiece == 0;
   const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
-  const int lowest = window > 0 ? max(0, ctx - window + 1) : 0;
+  const int lowest = chunk > 0 ? ctx / chunk * chunk : window > 0 ? max(0, ctx - window + 1) : 0;
   constexpr int GW = 64 / LK;                                // lane groups of a wave
   const int groups = nw * GW;
   for (int key0 = lowest + wave * GW + grp; key0 <= last_pos; key0 += groups * U) {
@@ -373,8 +386,8 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
       int slot = 0;
       if (ok) slot = page_shift >= 0 ? (table[key >> page_shift] << page_shift) + (key & (page_size - 1))
                                      : table[key / page_size] * page_size + key % page_size;
-      load_raw(kr[u], key_cache, ((int64_t)slot * kv_heads + g) * dim, pt * C, dim, ok, kvec);
-      load_raw(vr[u], value_cache, ((int64_t)slot * kv_heads + g) * vdim, pt * C, vdim, ok, vvec);
+      load_raw(kr[u], key_cache, (int64_t)slot * k_stride + (int64_t)g * dim, pt * C, dim, ok, kvec);
+      load_raw(vr[u], value_cache, (int64_t)slot * v_stride + (int64_t)g * vdim, pt * C, vdim, ok, vvec);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -387,7 +400,7 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
         for (int c = 0; c < C; ++c) s += qv[r][c] * kr[u].get(c);
         s = lanes_sum<LK>(s);
         if (softcap > 0.0f) s = softcap * fast_tanhf_(s * inv_cap);
-        const bool seen = key <= pos[r] && (window <= 0 || pos[r] - key < window);
+        const bool seen = key <= pos[r] && key >= low[r];
         if (!seen) s = -INFINITY;
         const float m_new = fmaxf(m_run[r], s);
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
@@ -433,7 +446,8 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
     const int tt = r / R, hh = r % R;
     float m_all = -INFINITY;
     for (int w = 0; w < nw; ++w) m_all = fmaxf(m_all, Ml[(w * RQ + r) * 2]);
-    float num = 0.0f, den = 0.0f;
+    if (sink) m_all = fmaxf(m_all, 0.0f);
+    float num = 0.0f, den = sink ? expf(-m_all) : 0.0f;
     for (int w = 0; w < nw; ++w) {
       const float f = fast_expf_(Ml[(w * RQ + r) * 2] - m_all);      // a wave that saw no key: 0
       den += f * Ml[(w * RQ + r) * 2 + 1];
@@ -450,7 +464,8 @@ template <typename T, int RQ, int C, int LK>
 int launch_capped_rows(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
                        int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
                        const int32_t* ctx_len, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
-                       float scale, float softcap, int window, hipStream_t stream) {
+                       float scale, float softcap, int window, int chunk, int sink, int64_t k_stride, int64_t v_stride,
+                       hipStream_t stream) {
   constexpr bool half = sizeof(typename Conv<T>::store_t) == 2;
   constexpr int U = RQ * C <= 32 ? (half ? 4 : 2) : (half ? 2 : 1);
   const int nw = 8;
@@ -467,7 +482,7 @@ int launch_capped_rows(void* out, const float* q, const void* key_cache, const v
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)num_seqs, (unsigned)kv_heads), dim3(64 * nw), lds_bytes, stream, out, q,
                      key_cache, value_cache, gate, gate_stride, block_tables, table_width, q_start, ctx_len, heads,
-                     kv_heads, dim, vdim, page_size, page_shift, scale, softcap, window);
+                     kv_heads, dim, vdim, page_size, page_shift, scale, softcap, window, chunk, sink, k_stride, v_stride);
   SW_CHECK_LAUNCH();
   return SW_OK;
 }
@@ -477,8 +492,8 @@ template <typename T>
 bool try_capped_rows(int* status, int rows_used, void* out, const float* q, const void* key_cache,
                      const void* value_cache, const void* gate, int64_t gate_stride, const int32_t* block_tables,
                      int table_width, const int32_t* q_start, const int32_t* ctx_len, int num_seqs, int heads,
-                     int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
-                     hipStream_t stream) {
+                     int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window, int chunk,
+                     int sink, int64_t k_stride, int64_t v_stride, hipStream_t stream) {
   if (rows_used > 8) return false;
   auto pow2 = [](int x) { return x <= 4 ? 4 : x <= 8 ? 8 : x <= 16 ? 16 : x <= 32 ? 32 : 64; };
   const int most = std::max(dim, vdim);
@@ -494,7 +509,8 @@ bool try_capped_rows(int* status, int rows_used, void* out, const float* q, cons
   if (rq == RQV && c == CV && lk == LKV) {                                                                              \
     *status = launch_capped_rows<T, RQV, CV, LKV>(out, q, key_cache, value_cache, gate, gate_stride, block_tables,      \
                                                   table_width, q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim,  \
-                                                  page_size, scale, softcap, window, stream);                           \
+                                                  page_size, scale, softcap, window, chunk, sink, k_stride, v_stride,   \
+                                                  stream);                                                              \
     return true;                                                                                                        \
   }
   SWM_ROWS_CASE(1, 4, 8) SWM_ROWS_CASE(1, 8, 8) SWM_ROWS_CASE(1, 16, 8) SWM_ROWS_CASE(1, 32, 8)
@@ -511,7 +527,7 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
                             int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
                             const int32_t* ctx_len, int64_t rows, int num_seqs, int max_query_len, int heads,
                             int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
-                            hipStream_t stream) {
+                            int chunk, int sink, int64_t k_stride, int64_t v_stride, hipStream_t stream) {
   const int R = heads / kv_heads;
   const int tpt = kQT / R;
   const int qstride = (dim + 31) / 32 * 32 + 4, ostride = NB * 32 + 1;
@@ -521,7 +537,7 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
     int status = SW_OK;
     if (try_capped_rows<T>(&status, rows_used, out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width,
                            q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim, page_size, scale, softcap, window,
-                           stream))
+                           chunk, sink, k_stride, v_stride, stream))
       return status;
   }
   auto lds_bytes = [&](int nw) {
@@ -548,27 +564,34 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
   const dim3 grid((unsigned)(split ? tiles : (tiles + nw - 1) / nw), (unsigned)kv_heads);
   hipLaunchKernelGGL(kernel, grid, dim3(64 * nw), lds_bytes(nw), stream, out, q, key_cache, value_cache, gate,
                      gate_stride, block_tables, table_width, q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim,
-                     page_size, scale, softcap, window, tpt, split ? 1 : 0, rows_used, page_shift);
+                     page_size, scale, softcap, window, chunk, sink, k_stride, v_stride, tpt, split ? 1 : 0, rows_used,
+                     page_shift);
   SW_CHECK_LAUNCH();
   return SW_OK;
 }
 
 }  // namespace swm
 
-extern "C" int swm_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
+extern "C" int swm_masked_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
                                     const void* gate, int64_t gate_stride, const int32_t* block_tables,
                                     int table_width, const int32_t* q_start, const int32_t* ctx_len, int64_t rows,
-                                    int num_seqs, int max_query_len, int heads, int kv_heads, int dim, int vdim, int page_size,
-                                    float scale, float softcap, int window, int act_dtype, void* stream) {
+                                    int num_seqs, int max_query_len, int heads, int kv_heads, int dim, int vdim,
+                                    int page_size, float scale, float softcap, int window, int chunk, int sink,
+                                    int64_t k_stride, int64_t v_stride, int act_dtype, void* stream) {
   using namespace swm;
   if (rows == 0 || num_seqs == 0) return SW_OK;
-  SW_CHECK_ARG(act_ok(act_dtype), "capped_attention: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(act_ok(act_dtype), "masked_attention: unsupported dtype %d", act_dtype);
   SW_CHECK_ARG(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && heads / kv_heads <= kQT,
-               "capped_attention: %d query heads on %d key/value heads (at most %d per key/value head)", heads, kv_heads,
+               "masked_attention: %d query heads on %d key/value heads (at most %d per key/value head)", heads, kv_heads,
                kQT);
-  SW_CHECK_ARG(dim > 0 && dim <= 256 && vdim > 0 && vdim <= 256 && page_size > 0 && table_width > 0 &&
-                   rows < (1ll << 31),
-               "capped_attention: key size %d, value size %d (at most 256 each)", dim, vdim);
+  SW_CHECK_ARG(dim > 0 && dim <= 32 * kMaxBlocks && vdim > 0 && vdim <= 32 * kMaxBlocks && page_size > 0 &&
+                   table_width > 0 && rows < (1ll << 31),
+               "masked_attention: key size %d, value size %d (at most %d each)", dim, vdim, 32 * kMaxBlocks);
+  SW_CHECK_ARG(!(window > 0 && chunk > 0) && window >= 0 && chunk >= 0,
+               "masked_attention: a sliding window (%d) or chunks (%d), not both", window, chunk);
+  SW_CHECK_ARG(k_stride >= (int64_t)kv_heads * dim && v_stride >= (int64_t)kv_heads * vdim,
+               "masked_attention: a cache slot of %lld / %lld elements cannot hold %d heads", (long long)k_stride,
+               (long long)v_stride, kv_heads);
   const int nvb = std::max((vdim + 31) / 32, (dim + 31) / 32);
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define SWM_CAPPED_CASE(N)                                                                                              \
@@ -576,7 +599,7 @@ extern "C" int swm_capped_attention(void* out, const float* q, const void* key_c
     SWM_DISPATCH_ACT(act_dtype, return (launch_capped_attention<T, N>(                                                  \
                                     out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width,       \
                                     q_start, ctx_len, rows, num_seqs, max_query_len, heads, kv_heads, dim, vdim,        \
-                                    page_size, scale, softcap, window, s)););                                                             \
+                                    page_size, scale, softcap, window, chunk, sink, k_stride, v_stride, s)););          \
     break;
   switch (nvb) {
     SWM_CAPPED_CASE(1)
@@ -587,7 +610,21 @@ extern "C" int swm_capped_attention(void* out, const float* q, const void* key_c
     SWM_CAPPED_CASE(6)
     SWM_CAPPED_CASE(7)
     SWM_CAPPED_CASE(8)
+    SWM_CAPPED_CASE(9)
+    SWM_CAPPED_CASE(10)
+    SWM_CAPPED_CASE(11)
+    SWM_CAPPED_CASE(12)
   }
 #undef SWM_CAPPED_CASE
   return SW_OK;
+}
+
+extern "C" int swm_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
+                                    const void* gate, int64_t gate_stride, const int32_t* block_tables,
+                                    int table_width, const int32_t* q_start, const int32_t* ctx_len, int64_t rows,
+                                    int num_seqs, int max_query_len, int heads, int kv_heads, int dim, int vdim, int page_size,
+                                    float scale, float softcap, int window, int act_dtype, void* stream) {
+  return swm_masked_attention(out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width, q_start,
+                              ctx_len, rows, num_seqs, max_query_len, heads, kv_heads, dim, vdim, page_size, scale,
+                              softcap, window, 0, 0, (int64_t)kv_heads * dim, (int64_t)kv_heads * vdim, act_dtype, stream);
 }

@@ -98,7 +98,8 @@ __global__ __launch_bounds__(kRowThreads) void qk_norm_cache_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(
     void* __restrict__ out, const float* __restrict__ o, const void* __restrict__ gate, int64_t gate_stride,
-    const float* __restrict__ weight, int weight_head_stride, float eps, int64_t rows, int heads, int vdim) {
+    const float* __restrict__ weight, int weight_head_stride, float eps, int64_t rows, int heads, int vdim,
+    int gate_silu) {
   const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (unit >= rows * heads) return;           // uniform over the wave
   const int lane = threadIdx.x & 63;
@@ -110,7 +111,8 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(
   ss = sw::wave_sum(ss);
   const float f = 1.0f / sqrtf(ss / (float)vdim + eps);
   for (int c = lane; c < vdim; c += 64) {
-    const float g = sigmoidf_(ld<T>(gate, t * gate_stride + h * vdim + c));
+    const float gv = ld<T>(gate, t * gate_stride + h * vdim + c);
+    const float g = gate_silu ? gv * sigmoidf_(gv) : sigmoidf_(gv);
     st<T>(out, (t * heads + h) * (int64_t)vdim + c, src[c] * f * weight[h * weight_head_stride + c] * g);
   }
 }
@@ -234,6 +236,13 @@ int swm_qk_norm_cache(float* q_out, const void* q, const void* k, const void* v,
 int swm_head_norm_gate(void* out, const float* o, const void* gate, int64_t gate_stride, const float* weight,
                        int weight_head_stride, float eps, int64_t rows, int heads, int vdim, int act_dtype,
                        void* stream) {
+  return swm_head_norm_gate_act(out, o, gate, gate_stride, weight, weight_head_stride, eps, rows, heads, vdim, 0,
+                                act_dtype, stream);
+}
+
+int swm_head_norm_gate_act(void* out, const float* o, const void* gate, int64_t gate_stride, const float* weight,
+                           int weight_head_stride, float eps, int64_t rows, int heads, int vdim, int gate_silu,
+                           int act_dtype, void* stream) {
   using namespace swm;
   if (rows == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "head_norm_gate: unsupported dtype %d", act_dtype);
@@ -241,7 +250,7 @@ int swm_head_norm_gate(void* out, const float* o, const void* gate, int64_t gate
   const unsigned blocks = (unsigned)((rows * heads + 3) / 4);
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(head_norm_gate_kernel<T>, dim3(blocks), dim3(256), 0,
                                                  static_cast<hipStream_t>(stream), out, o, gate, gate_stride, weight,
-                                                 weight_head_stride, eps, rows, heads, vdim););
+                                                 weight_head_stride, eps, rows, heads, vdim, gate_silu););
   SW_CHECK_LAUNCH();
   return SW_OK;
 }

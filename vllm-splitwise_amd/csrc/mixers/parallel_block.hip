@@ -71,10 +71,46 @@ __global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
     float* __restrict__ q_out, const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ v,
     int64_t in_stride, const int64_t* __restrict__ positions, const float* __restrict__ inv_freq, int rot_dims,
     void* __restrict__ key_cache, void* __restrict__ value_cache, const int64_t* __restrict__ slot_mapping, int heads,
-    int kv_heads, int dim, int vdim) {
+    int kv_heads, int dim, int vdim, int pair_halves) {
   const int64_t t = blockIdx.x;
   const int64_t row = t * in_stride;
   const float pos = (float)positions[t];
+  if (pair_halves) {
+    // coordinate i < rot_dims / 2 turns with coordinate i + rot_dims / 2; those from rot_dims on pass
+    const int hf = rot_dims / 2, units = dim - hf;            // a unit: one pair, or one passed-through coordinate
+    for (int e = threadIdx.x; e < heads * units; e += kPbThreads) {
+      const int h = e / units, u = e % units;
+      const int64_t src = row + h * dim, dst = t * (int64_t)heads * dim + h * dim;
+      if (u < hf) {
+        const float a = ld<T>(q, src + u), b = ld<T>(q, src + u + hf);
+        float s, c;
+        sincosf(pos * inv_freq[u], &s, &c);
+        q_out[dst + u] = a * c - b * s;
+        q_out[dst + u + hf] = b * c + a * s;
+      } else {
+        q_out[dst + u + hf] = ld<T>(q, src + u + hf);
+      }
+    }
+    if (k == nullptr) return;
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0) return;
+    for (int e = threadIdx.x; e < kv_heads * units; e += kPbThreads) {
+      const int h = e / units, u = e % units;
+      const int64_t src = row + h * dim, dst = slot * (int64_t)kv_heads * dim + h * dim;
+      if (u < hf) {
+        const float a = ld<T>(k, src + u), b = ld<T>(k, src + u + hf);
+        float s, c;
+        sincosf(pos * inv_freq[u], &s, &c);
+        st<T>(key_cache, dst + u, a * c - b * s);
+        st<T>(key_cache, dst + u + hf, b * c + a * s);
+      } else {
+        st<T>(key_cache, dst + u + hf, ld<T>(k, src + u + hf));
+      }
+    }
+    for (int e = threadIdx.x; e < kv_heads * vdim; e += kPbThreads)
+      st<T>(value_cache, slot * (int64_t)kv_heads * vdim + e, ld<T>(v, row + e));
+    return;
+  }
   const int half = rot_dims / 2, pairs = dim / 2;          // pairs beyond `half` pass through; so does an odd last one
   // queries
   for (int e = threadIdx.x; e < heads * pairs; e += kPbThreads) {
@@ -253,9 +289,9 @@ int swm_relu2(void* out, const void* in, int64_t in_stride, int64_t rows, int ff
 }
 
 int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, int64_t in_stride,
-                   const int64_t* positions, const float* inv_freq, int rot_dims, void* key_cache, void* value_cache,
-                   const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim, int vdim, int act_dtype,
-                   void* stream) {
+                   const int64_t* positions, const float* inv_freq, int rot_dims, int pair_halves, void* key_cache,
+                   void* value_cache, const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim,
+                   int vdim, int act_dtype, void* stream) {
   using namespace swm;
   if (rows == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "rope_cache: unsupported dtype %d", act_dtype);
@@ -268,7 +304,7 @@ int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, in
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(rope_cache_kernel<T>, dim3((unsigned)rows), dim3(kPbThreads), 0,
                                                  static_cast<hipStream_t>(stream), q_out, q, k, v, in_stride, positions,
                                                  inv_freq, rot_dims, key_cache, value_cache, slot_mapping, heads,
-                                                 kv_heads, dim, vdim););
+                                                 kv_heads, dim, vdim, pair_halves););
   SW_CHECK_LAUNCH();
   return SW_OK;
 }

@@ -18,7 +18,7 @@ import torch
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_PKG_DIR, "libsplitwise_mixers.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 SW_F32, SW_BF16 = 0, 2
 _ACT = {torch.float32: SW_F32, torch.bfloat16: SW_BF16}
@@ -42,11 +42,19 @@ _SIGNATURES = {
     "swm_stream_add_norm": [_p, _p, _l, _p, _l, _p, _p, _f, _f, _p, _l, _i, _i, _p],
     "swm_clamped_glu": [_p, _p, _l, _l, _i, _f, _f, _f, _i, _p],
     "swm_relu2": [_p, _p, _l, _l, _i, _i, _p],
-    "swm_rope_cache": [_p, _p, _p, _p, _l, _p, _p, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
+    "swm_rope_cache": [_p, _p, _p, _p, _l, _p, _p, _i, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
     "swm_group_router": [_p, _p, _p, _p, _l, _i, _i, _i, _i, _f, _p],
     "swm_group_pairs": [_p, _p, _p, _l, _i, _p],
     "swm_capped_attention": [_p, _p, _p, _p, _p, _l, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
                              _p],
+    "swm_masked_attention": [_p, _p, _p, _p, _p, _l, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
+                             _i, _l, _l, _i, _p],
+    "swm_gated_stream_step": [_p, _p, _l, _p, _l, _f, _p, _l, _p, _i, _p, _p, _p, _p, _l, _i, _i, _p],
+    "swm_poly_norm": [_p, _p, _l, _p, _f, _l, _i, _i, _p],
+    "swm_gate_mul": [_p, _p, _l, _l, _p, _l, _l, _i, _i, _i, _i, _p],
+    "swm_latent_rope_cache": [_p, _p, _l, _l, _p, _l, _l, _p, _l, _p, _f, _p, _p, _p, _p, _l, _i, _i, _i, _i, _p],
+    "swm_head_norm_gate_act": [_p, _p, _p, _l, _p, _i, _f, _l, _i, _i, _i, _i, _p],
+    "swm_gla": [_p, _p, _p, _p, _l, _p, _l, _p, _f, _f, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p],
     "swm_lightning": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
 }
 ACT_GELU, ACT_RELU2 = 0, 1
@@ -325,8 +333,9 @@ def general_delta(out: torch.Tensor, r: torch.Tensor, k: torch.Tensor, v: torch.
 
 
 def head_norm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, per_head_weight: bool,
-                   eps: float, heads: int, vdim: int) -> None:
-    """``per_head_weight``: weight is [heads * vdim]; otherwise [vdim], shared by the heads."""
+                   eps: float, heads: int, vdim: int, gate_silu: bool = False) -> None:
+    """``per_head_weight``: weight is [heads * vdim]; otherwise [vdim], shared by the heads.  ``gate_silu``: the
+    normed output is multiplied by gate * sigmoid(gate) instead of sigmoid(gate)."""
     _dev(out, o, gate, weight)
     _f32c(o, "o")
     _f32c(weight, "weight")
@@ -335,9 +344,10 @@ def head_norm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weigh
           and out.dtype == gate.dtype and weight.numel() == (heads * vdim if per_head_weight else vdim),
           "head_norm_gate: shapes")
     with _on_device_of(o):
-        _check(load_library().swm_head_norm_gate(out.data_ptr(), o.data_ptr(), gate.data_ptr(), _rows(gate, "gate"),
-                                                 weight.data_ptr(), vdim if per_head_weight else 0, eps, rows, heads,
-                                                 vdim, _act(out), _stream(o)))
+        _check(load_library().swm_head_norm_gate_act(out.data_ptr(), o.data_ptr(), gate.data_ptr(),
+                                                     _rows(gate, "gate"), weight.data_ptr(),
+                                                     vdim if per_head_weight else 0, eps, rows, heads, vdim,
+                                                     1 if gate_silu else 0, _act(out), _stream(o)))
 
 
 def expert_ffn(out: torch.Tensor, x: torch.Tensor, up: torch.Tensor, down: torch.Tensor, order: torch.Tensor,
@@ -424,9 +434,10 @@ def relu2(out: torch.Tensor, x: torch.Tensor) -> None:
 def rope_cache(q_out: torch.Tensor, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
                positions: torch.Tensor, inv_freq: Optional[torch.Tensor], heads: int, kv_heads: int, dim: int, vdim: int,
                key_cache: Optional[torch.Tensor], value_cache: Optional[torch.Tensor],
-               slot_mapping: Optional[torch.Tensor]) -> None:
+               slot_mapping: Optional[torch.Tensor], pair_halves: bool = False) -> None:
     """q, k, v: column ranges of ONE projection output.  q_out fp32 = rotated q; rotated k and v go to the caches
-    [pages, page, kv_heads * size] (k None: a layer that reads another layer's keys)."""
+    [pages, page, kv_heads * size] (k None: a layer that reads another layer's keys).  ``pair_halves``: coordinate i
+    turns with coordinate i + rot / 2 instead of neighbours (2i, 2i + 1)."""
     _dev(q_out, q, k, v, positions, inv_freq, key_cache, value_cache, slot_mapping)
     _f32c(q_out, "q_out")
     stride = _rows(q, "q")
@@ -454,7 +465,8 @@ def rope_cache(q_out: torch.Tensor, q: torch.Tensor, k: Optional[torch.Tensor], 
     with _on_device_of(q):
         _check(load_library().swm_rope_cache(
             q_out.data_ptr(), q.data_ptr(), _opt_ptr(k), _opt_ptr(v), stride, positions.data_ptr(),
-            _opt_ptr(inv_freq) if rot else None, rot, None if k is None else key_cache.data_ptr(),
+            _opt_ptr(inv_freq) if rot else None, rot, 1 if pair_halves else 0,
+            None if k is None else key_cache.data_ptr(),
             None if k is None else value_cache.data_ptr(), None if k is None else slot_mapping.data_ptr(), rows, heads,
             kv_heads, dim, vdim, _act(q), _stream(q)))
 
@@ -491,11 +503,14 @@ def group_pairs(chosen: torch.Tensor, experts: int):
     return order, start
 
 
-def capped_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+def capped_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor, value_cache: Optional[torch.Tensor],
                      gate: Optional[torch.Tensor], batch, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
-                     softcap: float = 0.0, window: int = 0) -> None:
+                     softcap: float = 0.0, window: int = 0, chunk: int = 0, sink: bool = False) -> None:
     """out [rows, heads * vdim] (cache dtype); q fp32 [rows, heads * dim]; caches [pages, page, kv_heads * size];
-    gate (None: no gate): a 2-D view [rows, heads * vdim] in the cache dtype."""
+    gate (None: no gate): a 2-D view [rows, heads * vdim] in the cache dtype.  ``window`` / ``chunk``: the mask (a
+    sliding window, or chunks counted from position 0; neither: plain causal); ``sink``: one more term exp(0) in the
+    softmax's denominator.  ``value_cache`` None: a token's values are the first kv_heads * vdim elements of its
+    key row (attention over a shared latent)."""
     _dev(out, q, key_cache, value_cache, gate)
     _f32c(q, "q")
     rows = q.shape[0]
@@ -504,20 +519,151 @@ def capped_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor
     _need(tables.dtype == torch.int32 and tables.is_contiguous() and tables.dim() == 2 and tables.shape[0] == n,
           "capped_attention: block tables")
     _need(q.shape[1] == heads * dim and out.shape == (rows, heads * vdim) and out.is_contiguous()
-          and out.dtype == key_cache.dtype == value_cache.dtype and key_cache.is_contiguous()
-          and value_cache.is_contiguous() and key_cache.shape[1:] == (value_cache.shape[1], kv_heads * dim)
-          and value_cache.shape[2] == kv_heads * vdim and key_cache.shape[0] == value_cache.shape[0],
-          "capped_attention: shapes")
+          and out.dtype == key_cache.dtype and key_cache.is_contiguous() and key_cache.dim() == 3
+          and key_cache.shape[2] >= kv_heads * dim, "capped_attention: shapes")
+    k_stride = key_cache.shape[2]
+    if value_cache is None:
+        _need(kv_heads * vdim <= k_stride and (kv_heads == 1 or vdim == dim),
+              "capped_attention: values inside the key rows need value size <= key size (equal with several heads)")
+        value_cache, v_stride = key_cache, k_stride
+    else:
+        _need(value_cache.dtype == out.dtype and value_cache.is_contiguous() and value_cache.dim() == 3
+              and value_cache.shape[:2] == key_cache.shape[:2] and value_cache.shape[2] >= kv_heads * vdim,
+              "capped_attention: value cache")
+        v_stride = value_cache.shape[2]
     _need(batch.max_pages_used <= tables.shape[1] and batch.max_page_id < key_cache.shape[0],
           "capped_attention: block tables exceed the cache")
     if gate is not None:
         _need(gate.shape == out.shape and gate.dtype == out.dtype, "capped_attention: gate")
     with _on_device_of(q):
-        _check(load_library().swm_capped_attention(
+        _check(load_library().swm_masked_attention(
             out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), _opt_ptr(gate),
             0 if gate is None else _rows(gate, "gate"), tables.data_ptr(), tables.shape[1], batch.q_start.data_ptr(),
             batch.ctx_len.data_ptr(), rows, n, int(getattr(batch, "max_query_len", 0) or 0), heads, kv_heads, dim, vdim,
-            key_cache.shape[1], scale, softcap, window, _act(out), _stream(q)))
+            key_cache.shape[1], scale, softcap, int(window), int(chunk), 1 if sink else 0, k_stride, v_stride,
+            _act(out), _stream(q)))
+
+
+def gated_stream_step(stream: torch.Tensor, y: Optional[torch.Tensor], gate: Optional[torch.Tensor], mult: float,
+                      history: Optional[torch.Tensor] = None, depth_weights: Optional[torch.Tensor] = None,
+                      norm=None, out: Optional[torch.Tensor] = None) -> None:
+    """stream (fp32 [rows, width], in place) += mult * y * sigmoid(gate) (y, gate: 2-D views in the activation
+    dtype; y None: nothing is added; gate None: no gate).  ``history`` fp32 [entries, rows, width] with
+    ``depth_weights`` fp32 [entries]: the sum is filed as the last entry and the stream becomes the entries'
+    weighted sum.  ``norm`` = (alpha [1], weight [width], bias [width]) fp32 with ``out``: out = tanh(alpha * stream)
+    * weight + bias in out's dtype."""
+    _dev(stream, y, gate, history, depth_weights, out)
+    _f32c(stream, "stream")
+    rows, width = stream.shape
+    act = out if out is not None else y
+    _need(act is not None or history is not None, "gated_stream_step: nothing to do")
+    if y is not None:
+        _need(y.shape == stream.shape and (gate is None or (gate.shape == stream.shape and gate.dtype == y.dtype)),
+              "gated_stream_step: addend and gate")
+    entries = 0
+    if history is not None:
+        _f32c(history, "history")
+        _f32c(depth_weights, "depth_weights")
+        entries = depth_weights.numel()
+        _need(history.dim() == 3 and history.shape[1:] == stream.shape and 1 <= entries <= history.shape[0],
+              "gated_stream_step: history")
+    alpha = weight = bias = None
+    if out is not None:
+        alpha, weight, bias = norm
+        for t, what in ((alpha, "alpha"), (weight, "norm weight"), (bias, "norm bias")):
+            _f32c(t, what)
+        _need(out.shape == stream.shape and out.is_contiguous() and alpha.numel() == 1 and weight.numel() == width
+              and bias.numel() == width and (y is None or y.dtype == out.dtype), "gated_stream_step: norm")
+    with _on_device_of(stream):
+        _check(load_library().swm_gated_stream_step(
+            stream.data_ptr(), _opt_ptr(y), 0 if y is None else _rows(y, "y"), _opt_ptr(gate),
+            0 if gate is None else _rows(gate, "gate"), mult, _opt_ptr(history), rows * width, _opt_ptr(depth_weights),
+            entries, _opt_ptr(alpha), _opt_ptr(weight), _opt_ptr(bias), _opt_ptr(out), rows, width,
+            SW_F32 if act is None else _act(act), _stream(stream)))
+
+
+def poly_norm(out: torch.Tensor, z: torch.Tensor, coef: torch.Tensor, eps: float) -> None:
+    """out [rows, ff] = c0 U(z) + c1 U(z^2) + c2 U(z^3) + c3 with U = division of a row by its root mean square;
+    coef fp32 [4]."""
+    _dev(out, z, coef)
+    _f32c(coef, "coef")
+    _need(out.is_contiguous() and out.shape == z.shape and out.dtype == z.dtype and coef.numel() == 4 and z.dim() == 2,
+          "poly_norm: shapes")
+    with _on_device_of(out):
+        _check(load_library().swm_poly_norm(out.data_ptr(), z.data_ptr(), _rows(z, "z"), coef.data_ptr(), eps,
+                                            z.shape[0], z.shape[1], _act(out), _stream(out)))
+
+
+def gate_mul(out: torch.Tensor, y: torch.Tensor, gate: torch.Tensor, silu: bool = False) -> None:
+    """out [rows, heads * size] = y * sigmoid(gate) (``silu``: y * gate * sigmoid(gate)); y is [rows, heads * size]
+    or a strided [rows, heads, size] view (e.g. the transpose of a batched product), gate a 2-D view."""
+    _dev(out, y, gate)
+    rows, n = out.shape
+    if y.dim() == 2:
+        y = y.unsqueeze(1)
+    _need(y.dim() == 3 and y.shape[0] == rows and y.shape[1] * y.shape[2] == n and y.stride(2) == 1
+          and gate.shape == out.shape and gate.dtype == out.dtype == y.dtype and out.is_contiguous(), "gate_mul: shapes")
+    with _on_device_of(out):
+        _check(load_library().swm_gate_mul(out.data_ptr(), y.data_ptr(), y.stride(0), y.stride(1), gate.data_ptr(),
+                                           _rows(gate, "gate"), rows, y.shape[1], y.shape[2], 1 if silu else 0,
+                                           _act(out), _stream(out)))
+
+
+def latent_rope_cache(q_out: torch.Tensor, q_latent: torch.Tensor, q_rot: torch.Tensor, down: Optional[torch.Tensor],
+                      norm_weight: Optional[torch.Tensor], eps: float, positions: torch.Tensor, inv_freq: torch.Tensor,
+                      cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor]) -> None:
+    """q_latent [rows, heads, rank], q_rot [rows, heads, rot]: strided views in the activation dtype; down [rows,
+    rank + rot]: a 2-D view; cache [pages, page, rank + rot].  q_out fp32 [rows, heads * (rank + rot)]."""
+    _dev(q_out, q_latent, q_rot, down, norm_weight, positions, inv_freq, cache, slot_mapping)
+    _f32c(q_out, "q_out")
+    rows, heads, rank = q_latent.shape
+    rot = q_rot.shape[2]
+    _need(q_rot.shape[:2] == (rows, heads) and q_latent.stride(2) == 1 and (rot == 0 or q_rot.stride(2) == 1)
+          and q_rot.dtype == q_latent.dtype and q_out.shape == (rows, heads * (rank + rot)), "latent_rope_cache: queries")
+    _need(positions.dtype == torch.int64 and positions.numel() == rows and positions.is_contiguous(),
+          "latent_rope_cache: positions must be int64 [rows]")
+    if rot:
+        _f32c(inv_freq, "inv_freq")
+        _need(2 * inv_freq.numel() == rot, "latent_rope_cache: one frequency per rotated pair")
+    if down is not None:
+        _f32c(norm_weight, "norm_weight")
+        _need(down.shape == (rows, rank + rot) and down.dtype == q_latent.dtype and norm_weight.numel() == rank
+              and cache.dtype == down.dtype and cache.is_contiguous() and cache.shape[-1] == rank + rot
+              and slot_mapping.dtype == torch.int64 and slot_mapping.numel() == rows and slot_mapping.is_contiguous(),
+              "latent_rope_cache: cache write")
+    with _on_device_of(q_out):
+        _check(load_library().swm_latent_rope_cache(
+            q_out.data_ptr(), q_latent.data_ptr(), q_latent.stride(0), q_latent.stride(1), q_rot.data_ptr(),
+            q_rot.stride(0), q_rot.stride(1), _opt_ptr(down), 0 if down is None else _rows(down, "down"),
+            _opt_ptr(norm_weight), eps, positions.data_ptr(), _opt_ptr(inv_freq) if rot else None,
+            None if down is None else cache.data_ptr(), None if down is None else slot_mapping.data_ptr(), rows, heads,
+            rank, rot, _act(q_latent), _stream(q_out)))
+
+
+def gla(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_pre: torch.Tensor,
+        decay_bias: Optional[torch.Tensor], tau: float, q_scale: float, state: torch.Tensor, batch, heads: int,
+        dim: int, vdim: int) -> None:
+    """out fp32 [rows, heads * vdim]; q, k, v: column ranges of one projection output; decay_pre [rows, heads * dim]
+    in the same dtype; decay_bias fp32 [heads * dim]; state fp32 [slots, heads, dim, vdim]."""
+    _dev(out, q, k, v, decay_pre, decay_bias, state)
+    for t, what in ((out, "out"), (state, "state")):
+        _f32c(t, what)
+    rows = q.shape[0]
+    n = _ragged_ok(batch, rows)
+    stride = _rows(q, "q")
+    _need(q.shape == (rows, heads * dim) and k.shape == q.shape and v.shape == (rows, heads * vdim)
+          and _rows(k, "k") == stride and _rows(v, "v") == stride and k.dtype == q.dtype and v.dtype == q.dtype
+          and decay_pre.shape == q.shape and decay_pre.dtype == q.dtype and out.shape == (rows, heads * vdim)
+          and state.shape[1:] == (heads, dim, vdim) and batch.max_state_slot < state.shape[0], "gla: shapes")
+    if decay_bias is not None:
+        _f32c(decay_bias, "decay_bias")
+        _need(decay_bias.numel() == heads * dim, "gla: one bias per head and key channel")
+    with _on_device_of(q):
+        _check(load_library().swm_gla(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride,
+                                      decay_pre.data_ptr(), _rows(decay_pre, "decay_pre"), _opt_ptr(decay_bias), tau,
+                                      q_scale, state.data_ptr(), batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
+                                      batch.state_slot.data_ptr(), rows, n, int(getattr(batch, "max_query_len", 0) or 0),
+                                      heads, dim, vdim, _act(q), _stream(q)))
 
 
 def lightning(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor,
@@ -550,4 +696,5 @@ ops = SimpleNamespace(expert_ffn=expert_ffn, ACT_GELU=ACT_GELU, ACT_RELU2=ACT_RE
     window_attention=window_attention, short_conv=short_conv, channel_delta=channel_delta,
     general_delta=general_delta, head_norm_gate=head_norm_gate, stream_add_norm=stream_add_norm,
     clamped_glu=clamped_glu, relu2=relu2, rope_cache=rope_cache, group_router=group_router, group_pairs=group_pairs,
-    capped_attention=capped_attention, lightning=lightning)
+    capped_attention=capped_attention, lightning=lightning, gated_stream_step=gated_stream_step, poly_norm=poly_norm,
+    gate_mul=gate_mul, latent_rope_cache=latent_rope_cache, gla=gla)

@@ -264,19 +264,23 @@ class WindowTalkingAttention(nn.Module):
 
 class CappedGatedAttention(nn.Module):
     """Causal softmax attention with grouped query heads over a paged cache, for models that want scores,
-    weights and positions in fp32:  partial rotary embedding on neighbouring pairs (frequencies given as a table,
-    angles from fp32 positions) on q and k, score = (q . k) * scale, optionally softcap * tanh(score / softcap),
-    optionally a sliding window, and optionally a sigmoid gate on the concatenated heads (the gate is a projection
-    of the same input as q).  Keys are cached AFTER rotation; a layer built with ``shares_kv`` has no key / value
-    projections and reads the cache of the layer it names with its own queries.  Caches are
-    [pages, page, kv_heads * size], token-major inside a page."""
+    weights and positions in fp32:  partial rotary embedding (frequencies given as a table, angles from fp32
+    positions; pairs are neighbours (2i, 2i + 1), or with ``pair_halves`` coordinates (i, i + rot / 2)) on q and k,
+    score = (q . k) * scale, optionally softcap * tanh(score / softcap), optionally a mask -- a sliding ``window``,
+    or ``chunk``: a position sees the earlier positions of its own chunk, chunks counted from position 0 --,
+    optionally one more term exp(0) in the softmax's denominator (``sink``: a key of score 0 without a value), and
+    optionally a sigmoid gate on the concatenated heads (the gate is a projection of the same input as q).  Keys are
+    cached AFTER rotation; a layer built with ``shares_kv`` has no key / value projections and reads the cache of the
+    layer it names with its own queries.  Caches are [pages, page, kv_heads * size], token-major inside a page."""
 
     def __init__(self, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, softcap: float = 0.0,
-                 inv_freq: Optional[torch.Tensor] = None, window: int = 0, shares_kv: bool = False) -> None:
+                 inv_freq: Optional[torch.Tensor] = None, window: int = 0, shares_kv: bool = False, chunk: int = 0,
+                 sink: bool = False, pair_halves: bool = False) -> None:
         super().__init__()
-        assert heads % kv_heads == 0
+        assert heads % kv_heads == 0 and not (window and chunk)
         self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
         self.scale, self.softcap, self.window, self.shares_kv = float(scale), float(softcap or 0.0), int(window), shares_kv
+        self.chunk, self.sink, self.pair_halves = int(chunk), bool(sink), bool(pair_halves)
         freqs = torch.zeros(0, dtype=torch.float32) if inv_freq is None else inv_freq.to(torch.float32)
         assert 2 * freqs.numel() <= dim
         self.register_buffer("inv_freq", freqs.clone(), persistent=False)     # a constant of the config, not a weight
@@ -293,11 +297,65 @@ class CappedGatedAttention(nn.Module):
         q32 = torch.empty(rows, self.heads * self.dim, dtype=torch.float32, device=q.device)
         if self.shares_kv:
             _C.mixer_ops.rope_cache(q32, q, None, None, positions, self.inv_freq, self.heads, self.kv_heads,
-                                    self.dim, self.vdim, None, None, None)
+                                    self.dim, self.vdim, None, None, None, self.pair_halves)
         else:
             _C.mixer_ops.rope_cache(q32, q, k, v, positions, self.inv_freq, self.heads, self.kv_heads, self.dim,
-                                    self.vdim, key_cache, value_cache, md.slot_mapping)
+                                    self.vdim, key_cache, value_cache, md.slot_mapping, self.pair_halves)
         out = torch.empty(rows, self.heads * self.vdim, dtype=q.dtype, device=q.device)
         _C.mixer_ops.capped_attention(out, q32, key_cache, value_cache, gate, md.ragged, self.heads, self.kv_heads,
-                                      self.dim, self.vdim, self.scale, self.softcap, self.window)
+                                      self.dim, self.vdim, self.scale, self.softcap, self.window, self.chunk, self.sink)
+        return out
+
+
+class LatentAttention(nn.Module):
+    """Softmax attention whose keys and values of ALL heads are linear maps of one small latent per token, plus one
+    rotated key part shared by the heads:
+        down = W_down x = [latent (rank) | shared key part (rot)],  c = rms_norm(latent) * w
+        key of head h = [U_k[h] c | rotate(shared part)],  value of head h = U_v[h] c
+        query of head h = [plain (dim) | rotated (rot)],   score = (q_plain . U_k[h] c + q_rot . k_rot) * scale
+    Only c and the rotated part are cached, one row of rank + rot numbers per token whatever the number of heads
+    ([pages, page, rank + rot]).  The up-projections never touch the cache: U_k[h] is applied to the QUERY
+    (q_plain^T U_k[h] is a vector of the latent's size, a batched GEMM over heads), attention then runs with one
+    shared key/value "head" whose key is the cache row and whose value is the row's first ``rank`` numbers, and
+    U_v[h] is applied to the attention's output (a second batched GEMM).  Optional sliding window and sigmoid gate
+    on the concatenated heads; scores, weights and sums are fp32."""
+
+    def __init__(self, heads: int, dim: int, rot: int, vdim: int, rank: int, scale: float, inv_freq: torch.Tensor,
+                 eps: float, dtype: torch.dtype, window: int = 0) -> None:
+        super().__init__()
+        self.heads, self.dim, self.rot, self.vdim, self.rank = heads, dim, rot, vdim, rank
+        self.scale, self.eps, self.window = float(scale), eps, int(window)
+        assert 2 * inv_freq.numel() == rot
+        self.register_buffer("inv_freq", inv_freq.to(torch.float32).clone(), persistent=False)
+        self.latent_norm = nn.Parameter(torch.ones(rank, dtype=torch.float32), requires_grad=False)
+        self.key_up = nn.Parameter(torch.zeros(heads, dim, rank, dtype=dtype), requires_grad=False)      # U_k[h]
+        self.value_up_t = nn.Parameter(torch.zeros(heads, rank, vdim, dtype=dtype), requires_grad=False)  # U_v[h]^T
+
+    def cache_shapes(self, block_size: int):
+        return [(block_size, self.rank + self.rot)]
+
+    def load_up_projections(self, key_up: torch.Tensor, value_up: torch.Tensor) -> None:
+        """key_up [heads * dim, rank], value_up [heads * vdim, rank], as a checkpoint stores them ([out, in])."""
+        self.key_up.data.copy_(key_up.view(self.heads, self.dim, self.rank))
+        self.value_up_t.data.copy_(value_up.view(self.heads, self.vdim, self.rank).transpose(1, 2))
+
+    def forward(self, q: torch.Tensor, down: torch.Tensor, gate: Optional[torch.Tensor], positions: torch.Tensor,
+                cache: torch.Tensor, md: InputMetadata) -> torch.Tensor:
+        """q [rows, heads * (dim + rot)], down [rows, rank + rot], gate [rows, heads * vdim]: column ranges of one
+        projection output.  -> [rows, heads * vdim]."""
+        rows, H, width = q.shape[0], self.heads, self.rank + self.rot
+        per_head = q.unflatten(1, (H, self.dim + self.rot))
+        q_latent = torch.bmm(per_head[:, :, :self.dim].transpose(0, 1), self.key_up)       # [heads, rows, rank]
+        q32 = torch.empty(rows, H * width, dtype=torch.float32, device=q.device)
+        _C.mixer_ops.latent_rope_cache(q32, q_latent.transpose(0, 1), per_head[:, :, self.dim:], down,
+                                       self.latent_norm.data, self.eps, positions, self.inv_freq, cache,
+                                       md.slot_mapping)
+        mixed = torch.empty(rows, H * self.rank, dtype=q.dtype, device=q.device)
+        _C.mixer_ops.capped_attention(mixed, q32, cache, None, None, md.ragged, H, 1, width, self.rank, self.scale,
+                                      0.0, self.window)
+        up = torch.bmm(mixed.unflatten(1, (H, self.rank)).transpose(0, 1), self.value_up_t)   # [heads, rows, vdim]
+        if gate is None:
+            return up.transpose(0, 1).reshape(rows, H * self.vdim)
+        out = torch.empty(rows, H * self.vdim, dtype=q.dtype, device=q.device)
+        _C.mixer_ops.gate_mul(out, up.transpose(0, 1), gate)
         return out

@@ -154,6 +154,70 @@ class OffsetRMSNorm(nn.Module):
         return self.add_norm(x, out_dtype)
 
 
+class DynamicTanhNorm(nn.Module):
+    """Element-wise norm without statistics of the row: out = tanh(alpha * x) * w + b, one number alpha, per-channel
+    w and b, all kept in fp32; reads an fp32 stream and writes activations.  ``gated_add_norm`` first takes a
+    sublayer's output into the stream through its gate (stream += mult * y * sigmoid(gate)) and, given the history of
+    layer outputs with the layer's depth weights, files the sum and replaces the stream by the weighted mix of all
+    entries, all in the one pass that also writes the norm."""
+
+    def __init__(self, width: int) -> None:
+        super().__init__()
+        self.alpha = nn.Parameter(torch.ones(1, dtype=torch.float32), requires_grad=False)
+        self.weight = nn.Parameter(torch.ones(width, dtype=torch.float32), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(width, dtype=torch.float32), requires_grad=False)
+
+    def _forward(self, x: torch.Tensor) -> torch.Tensor:
+        return torch.tanh(self.alpha * x.float()) * self.weight + self.bias
+
+    def gated_add_norm(self, stream: torch.Tensor, out_dtype: torch.dtype, y: Optional[torch.Tensor] = None,
+                       gate: Optional[torch.Tensor] = None, mult: float = 1.0,
+                       history: Optional[torch.Tensor] = None,
+                       depth_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+        out = torch.empty(stream.shape, dtype=out_dtype, device=stream.device)
+        _C.mixer_ops.gated_stream_step(stream, y, gate, mult, history, depth_weights,
+                                       (self.alpha.data, self.weight.data, self.bias.data), out)
+        return out
+
+    def forward(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        return self.gated_add_norm(x, out_dtype)
+
+    def load_named(self, state: dict, name: str) -> None:
+        self.weight.data.copy_(state[name].float())
+        self.alpha.data.copy_(state[name + ".alpha"].float().reshape(1))
+        self.bias.data.copy_(state[name + ".b"].float())
+
+
+class PolyNorm(nn.Module):
+    """Activation a U(z) + b U(z^2) + c U(z^3) + e with U(u) = u / sqrt(mean(u^2) + eps) over a row and the powers
+    taken element by element; the four numbers are one fp32 parameter."""
+
+    def __init__(self, eps: float) -> None:
+        super().__init__()
+        self.coef = nn.Parameter(torch.tensor([1.0, 0.0, 0.0, 0.0], dtype=torch.float32), requires_grad=False)
+        self.eps = eps
+
+    def _forward(self, z: torch.Tensor) -> torch.Tensor:
+        z = z.float()
+
+        def unit(u):
+            return u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + self.eps)
+        c = self.coef
+        return c[0] * unit(z) + c[1] * unit(z * z) + c[2] * unit(z * z * z) + c[3]
+
+    def forward(self, z: torch.Tensor) -> torch.Tensor:
+        """z: a 2-D view (a column range of a merged projection is fine)."""
+        out = torch.empty(z.shape, dtype=z.dtype, device=z.device)
+        _C.mixer_ops.poly_norm(out, z, self.coef.data, self.eps)
+        return out
+
+
+def rotary_frequencies(rot_dims: int, base: float) -> torch.Tensor:
+    """fp32 [rot_dims / 2]: f_i = base^(-2i / rot_dims), worked out in double precision, rounded once."""
+    return torch.tensor([float(base) ** (-2.0 * i / rot_dims) for i in range(rot_dims // 2)],
+                        dtype=torch.float64).to(torch.float32)
+
+
 def scaled_rotary_frequencies(rot_dims: int, base: float, scaling: Optional[dict] = None) -> torch.Tensor:
     """fp32 [rot_dims / 2]: f_i = base^(-2i / rot_dims), with long waves slowed down as Llama 3.1 does it
     (``scaling``: factor, low, high, original): a wavelength below original / high keeps f, one above original / low

@@ -15,6 +15,9 @@ Delta rule, per head, S [key size, value size] (keys index rows):
 Linear attention, per head, S [key size, value size]:
   ``LightningMixer``      S <- decay_h S + k v^T;  o = S^T q,  q, k, v = silu of their projections; the heads'
                           outputs are normed together, gated by a sigmoid and projected
+  ``GatedLinearAttentionMixer``  S <- diag(a) S + k v^T;  o = S^T q dim^(-1/2),  a = sigmoid(low-rank(h) + b)^(1 / tau)
+                          per head and key channel; each head's output is normed with a weight shared by the
+                          heads, gated by silu(gate) and projected
 """
 from typing import Dict, List, Sequence, Tuple
 
@@ -160,5 +163,57 @@ class LightningMixer(nn.Module):
 
     def load_named(self, w: Dict[str, torch.Tensor]) -> None:
         self.in_proj.weight.data.copy_(torch.cat([w["q"], w["k"], w["v"], w["g"]], 0))
+        self.o_proj.weight.data.copy_(w["o"])
+        self.out_norm.data.copy_(w["norm"].float())
+
+
+class GatedLinearAttentionMixer(nn.Module):
+    """Linear attention with a data-dependent decay per head and key channel, a_t = sigmoid(z_t)^(1 / tau) with z a
+    low-rank projection of the layer's input plus a bias.  q | k | v | gate | first decay factor (| ``extra_out``
+    more columns for the caller, e.g. a gate on the layer's output) are one GEMM; the decay's logarithm, the
+    recurrence and the output norm are fp32.  Each head's output gets an RMS norm over its value channels with ONE
+    weight [vdim] shared by the heads, times silu(gate), then the output projection."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay_rank: int, tau: float, eps: float,
+                 dtype: torch.dtype, linear_method=None, extra_out: int = 0) -> None:
+        super().__init__()
+        self.heads, self.dim, self.vdim, self.tau, self.eps = heads, dim, vdim, float(tau), eps
+        self.in_sizes = [heads * dim, heads * dim, heads * vdim, heads * vdim, decay_rank] + \
+            ([extra_out] if extra_out else [])
+        self.in_proj = MergedColumnParallelLinear(width, self.in_sizes, bool(extra_out), dtype, linear_method)
+        self.decay_up = ColumnParallelLinear(decay_rank, heads * dim, False, dtype, linear_method)
+        self.o_proj = RowParallelLinear(heads * vdim, width, False, dtype, linear_method)
+        self.decay_bias = _f32_param(heads * dim)
+        self.out_norm = nn.Parameter(torch.ones(vdim, dtype=torch.float32), requires_grad=False)
+
+    def state_shapes(self) -> List[Tuple[int, ...]]:
+        return [(self.heads, self.dim, self.vdim)]
+
+    def forward(self, h: torch.Tensor, state: List[torch.Tensor], md: InputMetadata):
+        """-> (output [rows, width], the ``extra_out`` columns of the input projection or None)."""
+        rows = h.shape[0]
+        proj = self.in_proj(h)
+        nk, nv, rank = self.heads * self.dim, self.heads * self.vdim, self.in_sizes[4]
+        lo = 2 * nk + 2 * nv
+        decay_pre = self.decay_up(proj[:, lo:lo + rank])
+        o = torch.empty(rows, nv, dtype=torch.float32, device=h.device)
+        _C.mixer_ops.gla(o, proj[:, :nk], proj[:, nk:2 * nk], proj[:, 2 * nk:2 * nk + nv], decay_pre,
+                         self.decay_bias.data, self.tau, self.dim ** -0.5, state[0], md.ragged, self.heads, self.dim,
+                         self.vdim)
+        gated = torch.empty(rows, nv, dtype=h.dtype, device=h.device)
+        _C.mixer_ops.head_norm_gate(gated, o, proj[:, 2 * nk + nv:lo], self.out_norm.data, False, self.eps, self.heads,
+                                    self.vdim, gate_silu=True)
+        extra = proj[:, lo + rank:] if len(self.in_sizes) > 5 else None
+        return self.o_proj(gated), extra
+
+    def load_named(self, w: Dict[str, torch.Tensor], extra: Dict[str, torch.Tensor] = None) -> None:
+        """``w``: q, k, v, g, a1, a2, a2.b, norm, o; ``extra``: weight / bias of the ``extra_out`` columns."""
+        parts = [w["q"], w["k"], w["v"], w["g"], w["a1"]] + ([extra["weight"]] if extra else [])
+        self.in_proj.weight.data.copy_(torch.cat(parts, 0))
+        if extra:
+            self.in_proj.bias.data.zero_()
+            self.in_proj.bias.data[-extra["bias"].numel():].copy_(extra["bias"])
+        self.decay_up.weight.data.copy_(w["a2"])
+        self.decay_bias.data.copy_(w["a2.b"].float())
         self.o_proj.weight.data.copy_(w["o"])
         self.out_norm.data.copy_(w["norm"].float())

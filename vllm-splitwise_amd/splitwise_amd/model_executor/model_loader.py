@@ -13,13 +13,14 @@ import torch
 import torch.nn as nn
 
 from ..config import ModelConfig
+from .models.lalasun import LalasunForCausalLM
 from .models.lapilorn import LapilornForCausalLM
 from .models.llama import LlamaForCausalLM
 from .models.nepevik import NepevikForCausalLM
 from .models.opt import OPTForCausalLM
 
 _ARCH = {"llama": LlamaForCausalLM, "opt": OPTForCausalLM, "nepevik": NepevikForCausalLM,
-         "lapilorn": LapilornForCausalLM}
+         "lapilorn": LapilornForCausalLM, "lalasun": LalasunForCausalLM}
 
 
 def architecture_class(name: str):
