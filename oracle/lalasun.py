@@ -12,7 +12,6 @@ With X_0 the embedding rows and X_(i+1) layer i's X, the next layer (or the outp
     sum_{j <= i+1} D_i[j] X_j        (D_i: the layer's i + 2 depth weights)
 Weights are [out, in] and applied as W u.  The logits come from a matrix of their own.
 """
-import math
 from typing import Dict, List
 
 import torch
@@ -24,10 +23,6 @@ def tanh_norm(u: torch.Tensor, a: torch.Tensor, w: torch.Tensor, b: torch.Tensor
 
 def rms_unit(u: torch.Tensor, eps: float) -> torch.Tensor:
     return u / torch.sqrt(u.pow(2).mean(-1, keepdim=True) + eps)
-
-
-def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
 def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
@@ -70,27 +65,47 @@ def rotate_halves(y: torch.Tensor, position: int, freqs: List[float]) -> torch.T
     return out
 
 
+def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, window: int = 0, chunk: int = 0,
+                     sink: bool = False, first_position: int = 0) -> torch.Tensor:
+    """q [n, H, d] at positions first_position ..; k [m, G, d], v [m, G, dv] from position 0.  -> [n, H, dv].
+    Query head a reads key/value head a // (H // G).  Position i sees j <= i, with ``window`` only i - j < window,
+    with ``chunk`` only j // chunk == i // chunk.  ``sink``: the weights are exp(s_j) / (1 + sum exp(s_j))."""
+    n, H, _ = q.shape
+    G = k.shape[1]
+    out = torch.zeros(n, H, v.shape[2], dtype=q.dtype)
+    for t in range(n):
+        pos = first_position + t
+        lo = max(0, pos - window + 1) if window else (pos // chunk) * chunk if chunk else 0
+        for a in range(H):
+            g = a // (H // G)
+            s = (k[lo:pos + 1, g] @ q[t, a]) * scale
+            if sink:
+                e = torch.exp(s)
+                p = e / (1.0 + e.sum())
+            else:
+                p = torch.softmax(s, 0)
+            out[t, a] = p @ v[lo:pos + 1, g]
+    return out
+
+
 def latent_attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: float) -> torch.Tensor:
     """Keys and values of all heads come from one small latent per token; one rotated key part is shared by the
     heads; sliding window; sigmoid gate on the heads' output."""
     n = h.shape[0]
     H, d, dr, dv, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
-    win = m["mask"]["size"]
     freqs = rotary_frequencies(m["rot"])
     assert m["rot"]["dims"] == dr
     q = (h @ w["q"].T).view(n, H, d + dr)
     down = h @ w["dkv"].T
     latent = rms_unit(down[:, :rank], eps) * w["dkv.norm"]
     k_rot = torch.stack([rotate_neighbours(down[t:t + 1, rank:], t, freqs)[0] for t in range(n)])
+    q_rot = torch.stack([rotate_neighbours(q[t, :, d:], t, freqs) for t in range(n)])
     k_plain = (latent @ w["uk"].T).view(n, H, d)
     v = (latent @ w["uv"].T).view(n, H, dv)
-    out = torch.zeros(n, H, dv, dtype=h.dtype)
-    for t in range(n):
-        q_rot = rotate_neighbours(q[t, :, d:], t, freqs)
-        lo = max(0, t - win + 1)
-        for a in range(H):
-            s = (k_plain[lo:t + 1, a] @ q[t, a, :d] + k_rot[lo:t + 1] @ q_rot[a]) * m["scale"]
-            out[t, a] = torch.softmax(s, 0) @ v[lo:t + 1, a]
+    # a head's key is its own plain part next to the part that all heads share
+    k_full = torch.cat([k_plain, k_rot.unsqueeze(1).expand(n, H, dr)], -1)
+    q_full = torch.cat([q[:, :, :d], q_rot], -1)
+    out = masked_attention(q_full, k_full, v, m["scale"], window=m["mask"]["size"])
     gate = torch.sigmoid(h @ w["g"].T)
     return (out.reshape(n, H * dv) * gate) @ w["o"].T
 
@@ -101,37 +116,41 @@ def chunked_sink_attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], m:
     n = h.shape[0]
     H, d, dv = m["heads"], m["dim"], m["vdim"]
     G = m.get("kv_heads", H)
-    size = m["mask"]["size"]
     freqs = rotary_frequencies(m["rot"])
     q = (h @ w["q"].T + w["q.b"]).view(n, H, d)
     k = (h @ w["k"].T + w["k.b"]).view(n, G, d)
     v = (h @ w["v"].T + w["v.b"]).view(n, G, dv)
     q = torch.stack([rotate_halves(q[t], t, freqs) for t in range(n)])
     k = torch.stack([rotate_halves(k[t], t, freqs) for t in range(n)])
-    out = torch.zeros(n, H, dv, dtype=h.dtype)
-    for t in range(n):
-        lo = (t // size) * size
-        for a in range(H):
-            g = a // (H // G)
-            e = torch.exp((k[lo:t + 1, g] @ q[t, a]) * m["scale"])
-            out[t, a] = (e / (1.0 + e.sum())) @ v[lo:t + 1, g]
+    out = masked_attention(q, k, v, m["scale"], chunk=m["mask"]["size"], sink=True)
     return out.reshape(n, H * dv) @ w["o"].T + w["o.b"]
 
 
+def decayed_state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state=None):
+    """q, k, decay [n, H, d], v [n, H, dv]:  S <- diag(decay_t) S + k_t v_t^T;  o_t = S^T q_t.  -> (o [n, H, dv], S)."""
+    n, H, d = q.shape
+    S = torch.zeros(H, d, v.shape[2], dtype=q.dtype) if state is None else state.clone()
+    o = torch.zeros(n, H, v.shape[2], dtype=q.dtype)
+    for t in range(n):
+        S = decay[t].unsqueeze(-1) * S + k[t].unsqueeze(-1) * v[t].unsqueeze(-2)
+        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    return o, S
+
+
+def channel_decay(z: torch.Tensor, tau: float) -> torch.Tensor:
+    """sigmoid(z)^(1 / tau), through the logarithm."""
+    return torch.exp(torch.nn.functional.logsigmoid(z) / tau)
+
+
 def gla_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: float) -> torch.Tensor:
-    """S <- diag(decay_t) S + k_t v_t^T;  o_t = S^T q_t, decay_t = sigmoid(z_t)^(1 / tau) per head and key channel."""
+    """Gated linear attention: a decay per head and key channel from a low-rank projection of the input."""
     n = h.shape[0]
     H, d, dv = m["heads"], m["dim"], m["vdim"]
     q = (h @ w["q"].T).view(n, H, d) * d ** -0.5
     k = (h @ w["k"].T).view(n, H, d)
     v = (h @ w["v"].T).view(n, H, dv)
-    z = (h @ w["a1"].T) @ w["a2"].T + w["a2.b"]
-    decay = torch.exp(torch.nn.functional.logsigmoid(z) / m["tau"]).view(n, H, d)
-    S = torch.zeros(H, d, dv, dtype=h.dtype)
-    o = torch.zeros(n, H, dv, dtype=h.dtype)
-    for t in range(n):
-        S = decay[t].unsqueeze(-1) * S + k[t].unsqueeze(-1) * v[t].unsqueeze(-2)
-        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    decay = channel_decay((h @ w["a1"].T) @ w["a2"].T + w["a2.b"], m["tau"]).view(n, H, d)
+    o, _ = decayed_state_scan(q, k, v, decay)
     o = rms_unit(o, eps) * w["norm"]
     gate = h @ w["g"].T
     return (o.reshape(n, H * dv) * (gate * torch.sigmoid(gate))) @ w["o"].T
