@@ -116,7 +116,7 @@ def parse_args():
                          "stack of equal size (random weights), and the mixer kernels beside the like Llama kernels with "
                          "their distances from the roofline; one JSON line")
     ap.add_argument("--mixer-sizes", default="2k", help="with --mixers: comma-separated preset sizes (2k, 4k)")
-    ap.add_argument("--mixer-family", default="nepevik", choices=["nepevik", "lapilorn"],
+    ap.add_argument("--mixer-family", default="nepevik", choices=["nepevik", "lapilorn", "lalasun"],
                     help="with --mixers: the family of listed-layer decoders to measure beside Llama")
     ap.add_argument("--replica", default=None, help=argparse.SUPPRESS)          # set by the launcher
     ap.add_argument("--worker-cls", default=None, help=argparse.SUPPRESS)       # CPU dry runs of the launcher

@@ -247,11 +247,15 @@ int swm_head_norm_gate_act(void* out, const float* o, const void* gate, int64_t 
  * a_t = sigmoid(decay_pre + decay_bias)^(1 / tau), i.e. log a_t = logsigmoid(.) / tau, worked out in fp32.
  * q, k [rows, heads * dim], v [rows, heads * vdim]: act_dtype column ranges of one projection output (row stride
  * in_stride); decay_pre act_dtype [rows, heads * dim] (row stride decay_stride); decay_bias fp32 [heads * dim] (NULL:
- * none); state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim].  Key size up to 256. */
+ * none); state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim].  Key size up to 256.
+ * max_query_len: the most new tokens of any sequence (0: unknown).  Long runs are cut into segments that run side by
+ * side and are joined by a scan over their end states; `workspace` then holds swm_gla_workspace_floats() floats (0:
+ * the step has no long run; NULL: never cut). */
+int64_t swm_gla_workspace_floats(int64_t rows, int num_seqs, int max_query_len, int heads, int dim, int vdim);
 int swm_gla(float* out, const void* q, const void* k, const void* v, int64_t in_stride, const void* decay_pre,
             int64_t decay_stride, const float* decay_bias, float tau, float q_scale, float* state,
             const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows, int num_seqs,
-            int max_query_len, int heads, int dim, int vdim, int act_dtype, void* stream);
+            int max_query_len, int heads, int dim, int vdim, float* workspace, int act_dtype, void* stream);
 
 /* Linear attention with one decay per head:  S <- decay[h] S + k v^T;  o = S^T q, with q, k, v = silu of the given
  * projections (act_dtype, column ranges of one output with row stride in_stride; q, k [rows, heads * dim],

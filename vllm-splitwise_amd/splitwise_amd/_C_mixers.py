@@ -54,7 +54,7 @@ _SIGNATURES = {
     "swm_gate_mul": [_p, _p, _l, _l, _p, _l, _l, _i, _i, _i, _i, _p],
     "swm_latent_rope_cache": [_p, _p, _l, _l, _p, _l, _l, _p, _l, _p, _f, _p, _p, _p, _p, _l, _i, _i, _i, _i, _p],
     "swm_head_norm_gate_act": [_p, _p, _p, _l, _p, _i, _f, _l, _i, _i, _i, _i, _p],
-    "swm_gla": [_p, _p, _p, _p, _l, _p, _l, _p, _f, _f, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _i, _p],
+    "swm_gla": [_p, _p, _p, _p, _l, _p, _l, _p, _f, _f, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
     "swm_lightning": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
 }
 ACT_GELU, ACT_RELU2 = 0, 1
@@ -83,6 +83,8 @@ def load_library() -> ctypes.CDLL:
     lib.swm_abi_version.restype, lib.swm_abi_version.argtypes = _i, []
     lib.swm_lightning_workspace_floats.restype = _l
     lib.swm_lightning_workspace_floats.argtypes = [_l, _i, _i, _i, _i, _i]
+    lib.swm_gla_workspace_floats.restype = _l
+    lib.swm_gla_workspace_floats.argtypes = [_l, _i, _i, _i, _i, _i]
     if lib.swm_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{_LIB_PATH} implements interface version {lib.swm_abi_version()}, this binding needs "
                            f"{ABI_VERSION}: rebuild it (`make -C vllm-splitwise_amd mixers`)")
@@ -658,12 +660,15 @@ def gla(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, de
     if decay_bias is not None:
         _f32c(decay_bias, "decay_bias")
         _need(decay_bias.numel() == heads * dim, "gla: one bias per head and key channel")
+    longest = int(getattr(batch, "max_query_len", 0) or 0)
     with _on_device_of(q):
-        _check(load_library().swm_gla(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride,
-                                      decay_pre.data_ptr(), _rows(decay_pre, "decay_pre"), _opt_ptr(decay_bias), tau,
-                                      q_scale, state.data_ptr(), batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
-                                      batch.state_slot.data_ptr(), rows, n, int(getattr(batch, "max_query_len", 0) or 0),
-                                      heads, dim, vdim, _act(q), _stream(q)))
+        lib = load_library()
+        need = lib.swm_gla_workspace_floats(rows, n, longest, heads, dim, vdim)
+        work = torch.empty(need, dtype=torch.float32, device=q.device) if need > 0 else None
+        _check(lib.swm_gla(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride, decay_pre.data_ptr(),
+                           _rows(decay_pre, "decay_pre"), _opt_ptr(decay_bias), tau, q_scale, state.data_ptr(),
+                           batch.q_start.data_ptr(), batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), rows, n,
+                           longest, heads, dim, vdim, _opt_ptr(work), _act(q), _stream(q)))
 
 
 def lightning(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor,

@@ -96,6 +96,34 @@ _LAPILORN_PRESETS = {
     "lapilorn-2k": (2048, 2, 16, 4, 32, 2, 1024),
     "lapilorn-4k": (4096, 2, 32, 8, 32, 2, 2048),
 }
+def _lalasun_preset(width: int, repeats: int, heads: int, kv_heads: int, ff: int) -> dict:
+    """A Lalasun stack of layer sizes that resemble a served model's: per repeat a gated-linear-attention layer, two
+    latent-attention layers (a 192-wide latent plus 64 rotated coordinates per token, window 1024), an attention layer
+    with grouped heads over chunks of 1024, and another gated-linear-attention layer, each with a dense feed-forward."""
+    d = width // heads
+    gla = {"heads": heads, "dim": d // 2, "vdim": d, "tau": 16.0, "decay_rank": 16}
+    latent = {"heads": heads, "dim": d // 2, "rot_dim": 64, "vdim": d, "kv_rank": 192, "scale": (d // 2 + 64) ** -0.5,
+              "mask": {"size": 1024}, "rot": {"base": 1000000.0, "dims": 64}}
+    attn = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024},
+            "rot": {"base": 500000.0, "dims": d}}
+    dense = {"kind": "dense", "ff": ff}
+    layers = []
+    for _ in range(repeats):
+        layers += [{"type": "gla", "mixer": dict(gla), "mlp": dense},
+                   {"type": "latent_attention", "mixer": dict(latent), "mlp": dense},
+                   {"type": "latent_attention", "mixer": dict(latent), "mlp": dense},
+                   {"type": "attention", "mixer": dict(attn), "mlp": dense},
+                   {"type": "gla", "mixer": dict(gla), "mlp": dense}]
+    from .model_executor.models.lalasun import normalize_config
+    return normalize_config({"architecture": "Lalasun", "layers": layers, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+                             "vocab": 32000, "width": width})
+
+
+_LALASUN_PRESETS = {
+    # name: (width, repeats of the 5-layer pattern, heads, kv heads, feed-forward size)
+    "lalasun-2k": (2048, 2, 16, 4, 4224),          # up + down of 4224 = gate + up + down of 2816
+    "lalasun-4k": (4096, 2, 32, 8, 8448),
+}
 # Llama stacks of the same width, depth and active feed-forward size, to measure the above against
 MODEL_PRESETS.update({
     "llama-2k": dict(architecture="llama", vocab_size=32000, hidden_size=2048, num_hidden_layers=10,
@@ -156,6 +184,8 @@ class ModelConfig:
             return _nepevik_preset(*_NEPEVIK_PRESETS[name])
         if name in _LAPILORN_PRESETS:
             return _lapilorn_preset(*_LAPILORN_PRESETS[name])
+        if name in _LALASUN_PRESETS:
+            return _lalasun_preset(*_LALASUN_PRESETS[name])
         cfg_path = os.path.join(model, "config.json")
         if os.path.isfile(cfg_path):
             with open(cfg_path) as f:

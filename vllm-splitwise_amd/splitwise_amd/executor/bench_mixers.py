@@ -1,4 +1,4 @@
-"""Throughput of a Nepevik (or Lapilorn) stack beside a Llama stack of the same width, depth and active feed-forward size
+"""Throughput of a Nepevik (or Lapilorn, or Lalasun) stack beside a Llama stack of the same width, depth and active feed-forward size
 (random weights), and every mixer kernel beside the like kernel of the Llama path with their distances from
 the roofline.  ``bench.py --mixers`` prints the result as one JSON line.
 
@@ -398,6 +398,142 @@ def kernel_table_lapilorn(width: int = 2048, heads: int = 16, kv_heads: int = 4,
     return rows
 
 
+@torch.inference_mode()
+def kernel_table_lalasun(width: int = 2048, heads: int = 16, kv_heads: int = 4, prefill_rows: int = 4096,
+                         decode_seqs: int = 64, decode_ctx: int = 2047, rank: int = 192, rot: int = 64, span: int = 1024,
+                         ff: int = 4224, depth: int = 6) -> List[dict]:
+    """The kernels of the Lalasun layers beside their like: the attention kernel with a chunk mask and a sink, and
+    over a shared latent, beside the same kernel as Lapilorn calls it (plain causal, grouped heads); the recurrence
+    with a decay per key channel beside the one with a decay per head; the gated stream step beside the fused add +
+    RMS norm; PolyNorm beside the clamped gated unit."""
+    from .. import _C
+    dev, bf = torch.device("cuda"), torch.bfloat16
+    d = width // heads
+    page = 16
+    rows: List[dict] = []
+    scale = d ** -0.5
+    for phase, seqs in (("prefill", [(0, prefill_rows // 2, 0, None), (0, prefill_rows // 2, 1, None)]),
+                        ("decode", [(decode_ctx, 1, i, None) for i in range(decode_seqs)])):
+        total_pages, laid = 0, []
+        for ctx, n, slot, _ in seqs:
+            pages = -(-(ctx + n) // page)
+            laid.append((ctx, n, slot, list(range(total_pages, total_pages + pages))))
+            total_pages += pages
+        batch = _ragged(laid, dev)
+        T, B = sum(s[1] for s in laid), len(laid)
+
+        def seen(limit_kind):
+            """(query, key) pairs and distinct keys read under a mask."""
+            pairs = keys = 0
+            for c, n, _, _ in laid:
+                for i in range(c, c + n):
+                    lo = 0 if limit_kind == "all" else i // span * span if limit_kind == "chunk" else max(0, i - span + 1)
+                    pairs += i - lo + 1
+                first = c if n == 1 else 0
+                lo = 0 if limit_kind == "all" else first // span * span if limit_kind == "chunk" else max(0, first - span + 1)
+                keys += c + n - lo
+            return pairs, keys
+        # ---------------------------------------------------------------- attention, grouped heads
+        kc = torch.randn(total_pages, page, kv_heads * d, device=dev).to(bf)
+        vc = torch.randn(total_pages, page, kv_heads * d, device=dev).to(bf)
+        q = torch.randn(T, heads * d, device=dev)
+        out = torch.empty(T, heads * d, dtype=bf, device=dev)
+        for name, kind, kw, like in (("masked attention (chunks of %d, sink)" % span, "chunk", dict(chunk=span, sink=True), ""),
+                                     ("capped_attention as Lapilorn runs it (causal, no cap)", "all", {}, "masked attention")):
+            t = _time(lambda: _C.mixer_ops.capped_attention(out, q, kc, vc, None, batch, heads, kv_heads, d, d, scale, 0.0, 0, **kw))
+            pairs, keys = seen(kind)
+            rows.append(_row(name, phase, t, keys * kv_heads * d * 2 * 2 + T * heads * d * (4 + 2), 4.0 * pairs * heads * d,
+                             VALU_F32, like=like))
+        # ---------------------------------------------------------------- attention over a shared latent
+        row = rank + rot
+        lc = torch.randn(total_pages, page, row, device=dev).to(bf)
+        ql = torch.randn(T, heads * row, device=dev)
+        lout = torch.empty(T, heads * rank, dtype=bf, device=dev)
+        t = _time(lambda: _C.mixer_ops.capped_attention(lout, ql, lc, None, None, batch, heads, 1, row, rank, scale, 0.0, span))
+        pairs, keys = seen("window")
+        rows.append(_row("latent attention (one %d-wide row per token, window %d)" % (row, span), phase, t,
+                         keys * row * 2 + T * heads * (row * 4 + rank * 2), 2.0 * pairs * heads * (row + rank), VALU_F32,
+                         like="capped_attention"))
+        # ---------------------------------------------------------------- rotation and cache writes
+        pos = torch.cat([torch.arange(c, c + n) for c, n, _, _ in laid]).to(dev)
+        slots = torch.cat([torch.tensor([tb[p // page] * page + p % page for p in range(c, c + n)])
+                           for c, n, _, tb in laid]).to(dev)
+        proj = torch.randn(T, (heads + 2 * kv_heads) * d, device=dev).to(bf)
+        inv = torch.rand(d // 2, device=dev)
+        q32 = torch.empty(T, heads * d, device=dev)
+        for name, halves, like in (("rope_cache, pairs (i, i + d/2)", True, ""), ("rope_cache, neighbouring pairs", False, "rope_cache")):
+            t = _time(lambda: _C.mixer_ops.rope_cache(q32, proj[:, :heads * d], proj[:, heads * d:(heads + kv_heads) * d],
+                                                      proj[:, (heads + kv_heads) * d:], pos, inv, heads, kv_heads, d, d, kc,
+                                                      vc, slots, halves))
+            rows.append(_row(name, phase, t, T * ((heads + 2 * kv_heads) * d * 2 + heads * d * 4 + 2 * kv_heads * d * 2),
+                             6.0 * T * heads * d, VALU_F32, like=like))
+        q_lat = torch.randn(heads, T, rank, device=dev).to(bf)
+        lproj = torch.randn(T, heads * (d // 2 + rot) + row, device=dev).to(bf)
+        qrot = lproj[:, :heads * (d // 2 + rot)].unflatten(1, (heads, d // 2 + rot))[:, :, d // 2:]
+        wl = torch.ones(rank, device=dev)
+        invl = torch.rand(rot // 2, device=dev)
+        t = _time(lambda: _C.mixer_ops.latent_rope_cache(ql, q_lat.transpose(0, 1), qrot, lproj[:, heads * (d // 2 + rot):], wl,
+                                                         1e-6, pos, invl, lc, slots))
+        rows.append(_row("latent_rope_cache (latent norm, rotation, query layout)", phase, t,
+                         T * (heads * (rank + rot) * (2 + 4) + row * 2 * 2), 6.0 * T * heads * rot, VALU_F32, like="rope_cache"))
+        # ---------------------------------------------------------------- recurrences
+        dk = d // 2
+        lseqs = [(c, n, i, []) for i, (c, n, _, _) in enumerate(laid)]
+        lbatch = _ragged(lseqs, dev)
+        gproj = torch.randn(T, heads * (2 * dk + d), device=dev).to(bf)
+        zpre = torch.randn(T, heads * dk, device=dev).to(bf)
+        zbias = torch.full((heads * dk,), 2.0, device=dev)
+        state = torch.zeros(max(B, 2), heads, dk, d, device=dev)
+        go = torch.empty(T, heads * d, device=dev)
+        t = _time(lambda: _C.mixer_ops.gla(go, gproj[:, :heads * dk], gproj[:, heads * dk:2 * heads * dk],
+                                           gproj[:, 2 * heads * dk:], zpre, zbias, 16.0, dk ** -0.5, state, lbatch, heads, dk, d))
+        chunk = 32
+        gflops = T * heads * (2.0 * chunk * dk + 2.0 * chunk * d + 4.0 * dk * d)
+        gbytes = T * heads * ((3 * dk + d) * 2 + d * 4) + 2 * B * heads * dk * d * 4
+        rows.append(_row("gla (decay per key channel)", phase, t, gbytes, gflops, VALU_F32))
+        decay = torch.full((heads,), 0.97, device=dev)
+        t2 = _time(lambda: _C.mixer_ops.lightning(go, gproj[:, :heads * dk], gproj[:, heads * dk:2 * heads * dk],
+                                                  gproj[:, 2 * heads * dk:], decay, state, lbatch, heads, dk, d))
+        rows.append(_row("Lapilorn lightning (decay per head), same sizes", phase, t2,
+                         T * heads * ((2 * dk + d) * 2 + d * 4) + 2 * B * heads * dk * d * 4, gflops, VALU_F32, like="gla"))
+        gate = torch.randn(T, heads * d, device=dev).to(bf)
+        gated = torch.empty(T, heads * d, dtype=bf, device=dev)
+        wn = torch.ones(d, device=dev)
+        t = _time(lambda: _C.mixer_ops.head_norm_gate(gated, go, gate, wn, False, 1e-6, heads, d, gate_silu=True))
+        rows.append(_row("head_norm_gate (per head, silu gate)", phase, t, T * heads * d * (4 + 2 + 2), 8.0 * T * heads * d, VALU_F32))
+        up = torch.randn(heads, T, d, device=dev).to(bf)
+        t = _time(lambda: _C.mixer_ops.gate_mul(gated, up.transpose(0, 1), gate))
+        rows.append(_row("gate_mul (heads of a batched product, sigmoid gate)", phase, t, T * heads * d * 2 * 3, 4.0 * T * heads * d,
+                         VALU_F32))
+        # ---------------------------------------------------------------- stream steps
+        stream = torch.randn(T, width, device=dev)
+        y = torch.randn(T, 2 * width, device=dev).to(bf)
+        hist = torch.randn(depth, T, width, device=dev)
+        dw = torch.rand(depth, device=dev)
+        norm = (torch.full((1,), 0.5, device=dev), torch.ones(width, device=dev), torch.zeros(width, device=dev))
+        hout = torch.empty(T, width, dtype=bf, device=dev)
+        t = _time(lambda: _C.mixer_ops.gated_stream_step(stream, y[:, :width], y[:, width:], 0.5, None, None, norm, hout))
+        rows.append(_row("gated_stream_step (gated add + tanh norm)", phase, t, T * width * (4 + 4 + 2 + 2 + 2), 10.0 * T * width, VALU_F32))
+        t = _time(lambda: _C.mixer_ops.gated_stream_step(stream, y[:, :width], y[:, width:], 0.5, hist, dw, norm, hout))
+        rows.append(_row("gated_stream_step (+ history of %d layers mixed)" % depth, phase, t,
+                         T * width * (4 + 4 + 2 + 2 + 2 + 4 * depth), (10.0 + 2 * depth) * T * width, VALU_F32))
+        a = torch.randn(T, width, device=dev).to(bf)
+        wgt = torch.zeros(width, device=dev)
+        t2 = _time(lambda: _C.mixer_ops.stream_add_norm(stream, wgt, 1.0, 1e-6, hout, a, a, None))
+        rows.append(_row("Lapilorn stream_add_norm (two addends)", phase, t2, T * width * (4 + 4 + 2 + 2 + 2), 6.0 * T * width, VALU_F32,
+                         like="gated_stream_step"))
+        # ---------------------------------------------------------------- feed-forward activation
+        z = torch.randn(T, ff + width, device=dev).to(bf)
+        act = torch.empty(T, ff, dtype=bf, device=dev)
+        coef = torch.tensor([1.0, 0.3, 0.1, 0.0], device=dev)
+        t = _time(lambda: _C.mixer_ops.poly_norm(act, z[:, :ff], coef, 1e-6))
+        rows.append(_row("poly_norm", phase, t, T * ff * 2 * 2, 14.0 * T * ff, VALU_F32))
+        gu = torch.randn(T, 2 * ff, device=dev).to(bf)
+        t2 = _time(lambda: _C.mixer_ops.clamped_glu(act, gu, 1.702, 7.0, 1.0))
+        rows.append(_row("Lapilorn clamped_glu", phase, t2, T * ff * 3 * 2, 8.0 * T * ff, VALU_F32, like="poly_norm"))
+    return rows
+
+
 def run(sizes=("2k",), with_kernels: bool = True, family: str = "nepevik") -> dict:
     result = {"family": family, "engine": {}, "kernels": {}}
     for size in sizes:
@@ -406,5 +542,6 @@ def run(sizes=("2k",), with_kernels: bool = True, family: str = "nepevik") -> di
             pair[name] = {k: round(v, 2) for k, v in engine_throughput(f"{name}-{size}").items()}
         result["engine"][size] = pair
     if with_kernels:
-        result["kernels"]["2k"] = kernel_table() if family == "nepevik" else kernel_table_lapilorn()
+        table = {"nepevik": kernel_table, "lapilorn": kernel_table_lapilorn, "lalasun": kernel_table_lalasun}[family]
+        result["kernels"]["2k"] = table()
     return result
