@@ -199,12 +199,17 @@ int swm_capped_attention(void* out, const float* q, const void* key_cache, const
  * 0: every j <= i.  `sink` != 0: the softmax's denominator has one more term, exp(0) (a key of score 0 without a
  * value).  A cache slot (one token) holds k_stride / v_stride elements, of which key/value head g's begin at g * dim /
  * g * vdim: value_cache may point into the key cache (values that are a part of the key row).  Key and value sizes up
- * to 384. */
+ * to 384.  Steps of few rows per sequence and few sequences share a tile's keys out among several workgroups, joined
+ * by a second launch: `workspace` then holds swm_masked_attention_workspace_floats() floats (0: not such a step;
+ * NULL: never shared out). */
+int64_t swm_masked_attention_workspace_floats(int64_t rows, int num_seqs, int max_query_len, int heads, int kv_heads,
+                                              int vdim, int page_size, int table_width, int window, int chunk);
 int swm_masked_attention(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
                          int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
                          const int32_t* ctx_len, int64_t rows, int num_seqs, int max_query_len, int heads,
                          int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
-                         int chunk, int sink, int64_t k_stride, int64_t v_stride, int act_dtype, void* stream);
+                         int chunk, int sink, int64_t k_stride, int64_t v_stride, float* workspace, int act_dtype,
+                         void* stream);
 
 /* ---- layers whose sublayer outputs enter an fp32 stream through a gate, with a mix over all earlier layers ---- */
 

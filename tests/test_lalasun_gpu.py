@@ -267,7 +267,7 @@ def test_chunked_attention_with_a_sink(H, G, d, dv, page, mode, cache_dtype, chu
 
 
 @pytest.mark.parametrize("H,rank,rot,page", [(3, 20, 4, 16), (4, 64, 16, 16), (2, 130, 6, 8), (1, 8, 2, 32), (8, 40, 8, 16),
-                                             (2, 288, 32, 16)])
+                                             (2, 288, 32, 16), (16, 24, 8, 16)])
 @pytest.mark.parametrize("mode", ["prompt", "decode", "pairs", "portions"])
 @pytest.mark.parametrize("cache_dtype,window", [(torch.float32, 37), (torch.bfloat16, 37), (torch.float32, 0), (torch.float32, 1)])
 def test_attention_over_a_shared_latent(H, rank, rot, page, mode, cache_dtype, window):
@@ -292,6 +292,43 @@ def test_attention_over_a_shared_latent(H, rank, rot, page, mode, cache_dtype, w
     ops().capped_attention(out, qd, kc, None, None, batch, H, 1, d, rank, scale, 0.0, window)
     tol = dict(atol=3e-5, rtol=3e-5) if cache_dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
     torch.testing.assert_close(out.cpu().double(), want[rows], **tol)
+
+
+@pytest.mark.parametrize("cache_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["latent", "grouped"])
+def test_decode_steps_of_few_sequences_share_their_keys_among_workgroups(kind, cache_dtype):
+    """Three sequences with long contexts and sixteen query heads per key row: the keys of each are shared out among
+    several workgroups whose parts a second launch joins.  A far key towers, one part sees no key at all (a window),
+    and the sink and the gate are applied once, by the join."""
+    n, page, H = 1500, 16, 16
+    rank, rot = (40, 8) if kind == "latent" else (0, 0)
+    d, dv = (rank + rot, rank) if kind == "latent" else (24, 40)
+    rows = [n - 1, 1201, 700]
+    spikes = [(n - 1, 3, 0), (1201, 1201 - 99, H - 1), (700, 650, 5)]
+    q, k, v = _attention_case(H, 1, d, dv, n, spikes, seed=77)
+    if kind == "latent":
+        kc, vc, table = _paged(k.reshape(n, d), None, page, cache_dtype, seed=5)
+    else:
+        kc, vc, table = _paged(k.reshape(n, d), v.reshape(n, dv), page, cache_dtype, seed=5)
+    kk = torch.stack([kc.cpu().double()[table[t // page], t % page].view(1, d) for t in range(n)])
+    vv = kk[:, :, :rank] if kind == "latent" else torch.stack([vc.cpu().double()[table[t // page], t % page].view(1, dv) for t in range(n)])
+    gate = torch.randn(len(rows), H * dv + 3, generator=torch.Generator().manual_seed(2)).to(cache_dtype)[:, 3:]
+    batch = ragged([(t, 1, 0, table) for t in rows])
+    qd = q[rows].reshape(len(rows), H * d).contiguous().to(DEV)
+    from splitwise_amd import _C_mixers
+    for window, chunk, sink, use_gate in [(0, 0, False, False), (100, 0, False, True), (0, 0, True, True), (0, 1100, True, False)]:
+        need = _C_mixers.load_library().swm_masked_attention_workspace_floats(len(rows), len(rows), 1, H, 1, dv, page, len(table),
+                                                                              window, chunk)
+        assert (need > 0) == (window == 0)                      # a short window leaves too few keys to share out
+        want = torch.stack([oracle.masked_attention(q[t:t + 1].double(), kk, vv, 0.9, window=window, chunk=chunk, sink=sink,
+                                                    first_position=t)[0] for t in rows]).reshape(len(rows), H * dv)
+        if use_gate:
+            want = want * torch.sigmoid(gate.double())
+        out = torch.empty(len(rows), H * dv, dtype=cache_dtype, device=DEV)
+        ops().capped_attention(out, qd, kc, None if kind == "latent" else vc, gate.to(DEV) if use_gate else None, batch, H, 1, d, dv,
+                               0.9, 0.0, window, chunk, sink)
+        tol = dict(atol=3e-5, rtol=3e-5) if cache_dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(out.cpu().double(), want, **tol)
 
 
 def _run_gla(proj, sizes, bias, tau, state, steps, H, d, dv):

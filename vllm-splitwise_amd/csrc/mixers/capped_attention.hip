@@ -112,7 +112,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
     float scale, float softcap, int window, int chunk, int sink, int64_t k_stride, int64_t v_stride, int tpt, int split,
-    int rows_used, int page_shift) {
+    int rows_used, int page_shift, float* __restrict__ partial, int64_t total_rows) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int R = heads / kv_heads;
   const int dblocks = (dim + 31) / 32;
@@ -167,7 +167,8 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
   float m_run = -INFINITY, l_run = 0.0f;
 
   const bool vvec = is_pow2(NB) && vdim % NB == 0 && v_stride % NB == 0;
-  const int kstep = split ? nw : 1;
+  // split: the waves of a workgroup, and with gridDim.z > 1 the workgroups of a tile, share the key tiles out
+  const int kstep = split ? nw * (int)gridDim.z : 1;
   // cache slot of key k0 + qi of a tile (-1: beyond the tile's last key)
   auto slot_of = [&](int k0) {
     const int key = k0 + qi;
@@ -194,7 +195,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
   // up to 128 there are registers for a second set of keys: the NEXT tile's keys are asked for at the same time and
   // arrive during this tile; otherwise a tile's keys are asked for when the tile before it ends.
   constexpr bool kAhead = sizeof(typename Conv<T>::store_t) == 2 && NB <= 4;
-  int kt = tile_lo + (split ? wave : 0);
+  int kt = tile_lo + (split ? (int)blockIdx.z * nw + wave : 0);
   Raw<T, 16> kraw[NB];
   int slot_cur = -1, slot_next = -1;
   if (kt <= tile_hi) {
@@ -295,6 +296,28 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
       float m_all = -INFINITY;
       for (int w = 0; w < nw; ++w) m_all = fmaxf(m_all, Ml[(w * kQT + r) * 2]);
       if (sink) m_all = fmaxf(m_all, 0.0f);                  // one more term of score 0 that carries no value
+      if (partial != nullptr) {
+        // this workgroup saw a part of the keys: its maximum, denominator and unnormalised sums go to the scratch that
+        // the join kernel reads; the sink is the join's business
+        float m_part = -INFINITY;
+        for (int w = 0; w < nw; ++w) m_part = fmaxf(m_part, Ml[(w * kQT + r) * 2]);
+        float num = 0.0f, den = 0.0f;
+        if (m_part != -INFINITY)
+          for (int w = 0; w < nw; ++w) {
+            const float f = expf(Ml[(w * kQT + r) * 2] - m_part);
+            den += f * Ml[(w * kQT + r) * 2 + 1];
+            num += f * Oall[(w * rows_used + r) * ostride + c];
+          }
+        const int64_t pr = ((int64_t)blockIdx.z * total_rows + row0 + tt) * heads + g * R + hh;
+        float* ml = partial;
+        float* po = partial + (int64_t)gridDim.z * total_rows * heads * 2;
+        if (c == 0) {
+          ml[pr * 2] = m_part;
+          ml[pr * 2 + 1] = den;
+        }
+        po[pr * vdim + c] = num;
+        continue;
+      }
       float num = 0.0f, den = sink ? expf(-m_all) : 0.0f;
       for (int w = 0; w < nw; ++w) {
         const float f = expf(Ml[(w * kQT + r) * 2] - m_all);  // a wave that saw no key: exp(-inf) = 0
@@ -522,12 +545,60 @@ bool try_capped_rows(int* status, int rows_used, void* out, const float* q, cons
   return false;
 }
 
+// Joins the parts of a step whose keys were shared out among `parts` workgroups per tile: one workgroup per
+// (row, head), parts in a fixed order.
+template <typename T>
+__global__ __launch_bounds__(256) void capped_attention_join_kernel(
+    void* __restrict__ out, const float* __restrict__ partial, const void* __restrict__ gate, int64_t gate_stride,
+    int64_t total_rows, int heads, int vdim, int parts, int sink) {
+  const int64_t rh = blockIdx.x;                             // row * heads + head
+  const float* ml = partial;
+  const float* po = partial + (int64_t)parts * total_rows * heads * 2;
+  const int64_t part_stride = total_rows * heads;
+  float m_all = sink ? 0.0f : -INFINITY;
+  for (int z = 0; z < parts; ++z) m_all = fmaxf(m_all, ml[(z * part_stride + rh) * 2]);
+  float den = sink ? expf(-m_all) : 0.0f;
+  for (int z = 0; z < parts; ++z) {
+    const float m = ml[(z * part_stride + rh) * 2];
+    if (m != -INFINITY) den += expf(m - m_all) * ml[(z * part_stride + rh) * 2 + 1];
+  }
+  const int64_t t = rh / heads;
+  const int hd = (int)(rh % heads);
+  for (int c = threadIdx.x; c < vdim; c += blockDim.x) {
+    float num = 0.0f;
+    for (int z = 0; z < parts; ++z) {
+      const float m = ml[(z * part_stride + rh) * 2];
+      if (m != -INFINITY) num += expf(m - m_all) * po[(z * part_stride + rh) * vdim + c];
+    }
+    float v = num / den;
+    if (gate != nullptr) v *= sigmoidf_(ld<T>(gate, t * gate_stride + (int64_t)hd * vdim + c));
+    st<T>(out, rh * vdim + c, v);
+  }
+}
+
+// In how many parts the keys of a tile are shared out among workgroups: steps of few rows per sequence (decode steps)
+// of few sequences would otherwise leave most of the GPU idle.  most_keys: an upper bound on the keys a row sees.
+inline int key_parts(int num_seqs, int max_query_len, int heads, int kv_heads, int page_size, int table_width, int window,
+                     int chunk) {
+  const int R = heads / kv_heads, tpt = kQT / R;
+  if (max_query_len <= 0 || max_query_len > tpt || max_query_len * R <= 8) return 1;   // not the shared-keys loop
+  int64_t most_keys = (int64_t)page_size * table_width;
+  if (window > 0) most_keys = std::min<int64_t>(most_keys, window + max_query_len);
+  if (chunk > 0) most_keys = std::min<int64_t>(most_keys, chunk);
+  const int64_t tiles = (most_keys + kQT - 1) / kQT;
+  const int64_t groups = (int64_t)num_seqs * kv_heads;
+  int parts = 1;
+  while (parts < 16 && groups * parts * 2 <= 512 && tiles >= 8 * parts * 2) parts <<= 1;
+  return parts;
+}
+
 template <typename T, int NB>
 int launch_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
                             int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
                             const int32_t* ctx_len, int64_t rows, int num_seqs, int max_query_len, int heads,
                             int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
-                            int chunk, int sink, int64_t k_stride, int64_t v_stride, hipStream_t stream) {
+                            int chunk, int sink, int64_t k_stride, int64_t v_stride, float* workspace,
+                            hipStream_t stream) {
   const int R = heads / kv_heads;
   const int tpt = kQT / R;
   const int qstride = (dim + 31) / 32 * 32 + 4, ostride = NB * 32 + 1;
@@ -545,9 +616,13 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
                                 : (size_t)nw * kQT * std::max(qstride, ostride);
     return floats * sizeof(float);
   };
-  // two workgroups of a compute unit's 160 KB where the sizes allow it
+  const int parts = (split && workspace != nullptr)
+                        ? key_parts(num_seqs, max_query_len, heads, kv_heads, page_size, table_width, window, chunk) : 1;
+  // two workgroups of a compute unit's 160 KB where the sizes allow it; a launch that cannot fill the compute units
+  // twice anyway gives each workgroup as many waves as one unit's LDS holds
+  const bool few = split && (int64_t)num_seqs * kv_heads * parts <= 256;
   int nw = split ? 8 : 4;
-  while (nw > 1 && lds_bytes(nw) > 72 * 1024) nw >>= 1;
+  while (nw > 1 && lds_bytes(nw) > (few ? 150 : 72) * 1024) nw >>= 1;
   SW_CHECK_ARG(lds_bytes(nw) <= 160 * 1024, "capped_attention: key size %d with value size %d needs too much LDS", dim,
                vdim);
   auto kernel = capped_attention_kernel<T, NB>;
@@ -561,23 +636,36 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
     allowed = lds_bytes(nw);
   }
   const int64_t tiles = split ? num_seqs : (rows + tpt - 1) / tpt + num_seqs;
-  const dim3 grid((unsigned)(split ? tiles : (tiles + nw - 1) / nw), (unsigned)kv_heads);
+  const dim3 grid((unsigned)(split ? tiles : (tiles + nw - 1) / nw), (unsigned)kv_heads, (unsigned)parts);
   hipLaunchKernelGGL(kernel, grid, dim3(64 * nw), lds_bytes(nw), stream, out, q, key_cache, value_cache, gate,
                      gate_stride, block_tables, table_width, q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim,
                      page_size, scale, softcap, window, chunk, sink, k_stride, v_stride, tpt, split ? 1 : 0, rows_used,
-                     page_shift);
+                     page_shift, parts > 1 ? workspace : (float*)nullptr, rows);
   SW_CHECK_LAUNCH();
+  if (parts > 1) {
+    hipLaunchKernelGGL(capped_attention_join_kernel<T>, dim3((unsigned)(rows * heads)), dim3(vdim <= 64 ? 64 : 128), 0,
+                       stream, out, workspace, gate, gate_stride, rows, heads, vdim, parts, sink);
+    SW_CHECK_LAUNCH();
+  }
   return SW_OK;
 }
 
 }  // namespace swm
+
+extern "C" int64_t swm_masked_attention_workspace_floats(int64_t rows, int num_seqs, int max_query_len, int heads,
+                                                         int kv_heads, int vdim, int page_size, int table_width,
+                                                         int window, int chunk) {
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || heads / kv_heads > swm::kQT) return 0;
+  const int parts = swm::key_parts(num_seqs, max_query_len, heads, kv_heads, page_size, table_width, window, chunk);
+  return parts > 1 ? (int64_t)parts * rows * heads * (vdim + 2) : 0;
+}
 
 extern "C" int swm_masked_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
                                     const void* gate, int64_t gate_stride, const int32_t* block_tables,
                                     int table_width, const int32_t* q_start, const int32_t* ctx_len, int64_t rows,
                                     int num_seqs, int max_query_len, int heads, int kv_heads, int dim, int vdim,
                                     int page_size, float scale, float softcap, int window, int chunk, int sink,
-                                    int64_t k_stride, int64_t v_stride, int act_dtype, void* stream) {
+                                    int64_t k_stride, int64_t v_stride, float* workspace, int act_dtype, void* stream) {
   using namespace swm;
   if (rows == 0 || num_seqs == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "masked_attention: unsupported dtype %d", act_dtype);
@@ -599,7 +687,8 @@ extern "C" int swm_masked_attention(void* out, const float* q, const void* key_c
     SWM_DISPATCH_ACT(act_dtype, return (launch_capped_attention<T, N>(                                                  \
                                     out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width,       \
                                     q_start, ctx_len, rows, num_seqs, max_query_len, heads, kv_heads, dim, vdim,        \
-                                    page_size, scale, softcap, window, chunk, sink, k_stride, v_stride, s)););          \
+                                    page_size, scale, softcap, window, chunk, sink, k_stride, v_stride, workspace,      \
+                                    s)););                                                                              \
     break;
   switch (nvb) {
     SWM_CAPPED_CASE(1)
@@ -626,5 +715,6 @@ extern "C" int swm_capped_attention(void* out, const float* q, const void* key_c
                                     float scale, float softcap, int window, int act_dtype, void* stream) {
   return swm_masked_attention(out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width, q_start,
                               ctx_len, rows, num_seqs, max_query_len, heads, kv_heads, dim, vdim, page_size, scale,
-                              softcap, window, 0, 0, (int64_t)kv_heads * dim, (int64_t)kv_heads * vdim, act_dtype, stream);
+                              softcap, window, 0, 0, (int64_t)kv_heads * dim, (int64_t)kv_heads * vdim, nullptr, act_dtype,
+                              stream);
 }

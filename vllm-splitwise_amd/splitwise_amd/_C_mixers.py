@@ -48,7 +48,7 @@ _SIGNATURES = {
     "swm_capped_attention": [_p, _p, _p, _p, _p, _l, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
                              _p],
     "swm_masked_attention": [_p, _p, _p, _p, _p, _l, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
-                             _i, _l, _l, _i, _p],
+                             _i, _l, _l, _p, _i, _p],
     "swm_gated_stream_step": [_p, _p, _l, _p, _l, _f, _p, _l, _p, _i, _p, _p, _p, _p, _l, _i, _i, _p],
     "swm_poly_norm": [_p, _p, _l, _p, _f, _l, _i, _i, _p],
     "swm_gate_mul": [_p, _p, _l, _l, _p, _l, _l, _i, _i, _i, _i, _p],
@@ -83,6 +83,8 @@ def load_library() -> ctypes.CDLL:
     lib.swm_abi_version.restype, lib.swm_abi_version.argtypes = _i, []
     lib.swm_lightning_workspace_floats.restype = _l
     lib.swm_lightning_workspace_floats.argtypes = [_l, _i, _i, _i, _i, _i]
+    lib.swm_masked_attention_workspace_floats.restype = _l
+    lib.swm_masked_attention_workspace_floats.argtypes = [_l, _i, _i, _i, _i, _i, _i, _i, _i, _i]
     lib.swm_gla_workspace_floats.restype = _l
     lib.swm_gla_workspace_floats.argtypes = [_l, _i, _i, _i, _i, _i]
     if lib.swm_abi_version() != ABI_VERSION:
@@ -537,13 +539,17 @@ def capped_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor
           "capped_attention: block tables exceed the cache")
     if gate is not None:
         _need(gate.shape == out.shape and gate.dtype == out.dtype, "capped_attention: gate")
+    longest = int(getattr(batch, "max_query_len", 0) or 0)
     with _on_device_of(q):
-        _check(load_library().swm_masked_attention(
+        lib = load_library()
+        need = lib.swm_masked_attention_workspace_floats(rows, n, longest, heads, kv_heads, vdim, key_cache.shape[1],
+                                                         tables.shape[1], int(window), int(chunk))
+        work = torch.empty(need, dtype=torch.float32, device=q.device) if need > 0 else None
+        _check(lib.swm_masked_attention(
             out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), _opt_ptr(gate),
             0 if gate is None else _rows(gate, "gate"), tables.data_ptr(), tables.shape[1], batch.q_start.data_ptr(),
-            batch.ctx_len.data_ptr(), rows, n, int(getattr(batch, "max_query_len", 0) or 0), heads, kv_heads, dim, vdim,
-            key_cache.shape[1], scale, softcap, int(window), int(chunk), 1 if sink else 0, k_stride, v_stride,
-            _act(out), _stream(q)))
+            batch.ctx_len.data_ptr(), rows, n, longest, heads, kv_heads, dim, vdim, key_cache.shape[1], scale, softcap,
+            int(window), int(chunk), 1 if sink else 0, k_stride, v_stride, _opt_ptr(work), _act(out), _stream(q)))
 
 
 def gated_stream_step(stream: torch.Tensor, y: Optional[torch.Tensor], gate: Optional[torch.Tensor], mult: float,
