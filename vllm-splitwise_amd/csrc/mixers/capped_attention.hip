@@ -105,8 +105,13 @@ constexpr bool is_pow2(int n) { return n > 0 && (n & (n - 1)) == 0; }
 // split != 0 (steps in which no sequence brings more tokens than one tile holds, a decode step above all): a workgroup
 //   owns one tile and its waves share the keys out among them, joined through LDS (rows_used query rows are live).
 // split == 0: every wave owns a tile of its own and walks all of its keys; nothing is joined.
+// Up to 128 coordinates the kernel's registers fit two waves per SIMD (workgroups of up to 8 waves); beyond that a wave
+// needs more than 256 registers, so those instantiations are built for workgroups of at most 4 waves (one per SIMD, 512
+// registers each) instead of spilling.
+constexpr int max_waves_of(int nb) { return nb <= 4 ? 8 : 4; }
+
 template <typename T, int NB>
-__global__ __launch_bounds__(512) void capped_attention_kernel(
+__global__ __launch_bounds__(64 * max_waves_of(NB)) void capped_attention_kernel(
     void* __restrict__ out, const float* __restrict__ q, const void* __restrict__ key_cache,
     const void* __restrict__ value_cache, const void* __restrict__ gate, int64_t gate_stride,
     const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
@@ -257,7 +262,7 @@ __global__ __launch_bounds__(512) void capped_attention_kernel(
     // ---- O^T = alpha O^T + V^T P^T
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      if (b < vdim) {
+      if (b < vdim) {                                          // block b holds the channels NB * lane + b
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
 #pragma unroll
@@ -621,7 +626,7 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
   // two workgroups of a compute unit's 160 KB where the sizes allow it; a launch that cannot fill the compute units
   // twice anyway gives each workgroup as many waves as one unit's LDS holds
   const bool few = split && (int64_t)num_seqs * kv_heads * parts <= 256;
-  int nw = split ? 8 : 4;
+  int nw = split ? max_waves_of(NB) : 4;
   while (nw > 1 && lds_bytes(nw) > (few ? 150 : 72) * 1024) nw >>= 1;
   SW_CHECK_ARG(lds_bytes(nw) <= 160 * 1024, "capped_attention: key size %d with value size %d needs too much LDS", dim,
                vdim);
