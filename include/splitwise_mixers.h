@@ -199,7 +199,7 @@ int swm_capped_attention(void* out, const float* q, const void* key_cache, const
  * 0: every j <= i.  `sink` != 0: the softmax's denominator has one more term, exp(0) (a key of score 0 without a
  * value).  A cache slot (one token) holds k_stride / v_stride elements, of which key/value head g's begin at g * dim /
  * g * vdim: value_cache may point into the key cache (values that are a part of the key row).  Key and value sizes up
- * to 384.  Steps of few rows per sequence and few sequences share a tile's keys out among several workgroups, joined
+ * to 512.  Steps of few rows per sequence and few sequences share a tile's keys out among several workgroups, joined
  * by a second launch: `workspace` then holds swm_masked_attention_workspace_floats() floats (0: not such a step;
  * NULL: never shared out). */
 int64_t swm_masked_attention_workspace_floats(int64_t rows, int num_seqs, int max_query_len, int heads, int kv_heads,

@@ -267,7 +267,7 @@ def test_chunked_attention_with_a_sink(H, G, d, dv, page, mode, cache_dtype, chu
 
 
 @pytest.mark.parametrize("H,rank,rot,page", [(3, 20, 4, 16), (4, 64, 16, 16), (2, 130, 6, 8), (1, 8, 2, 32), (8, 40, 8, 16),
-                                             (2, 288, 32, 16), (16, 24, 8, 16)])
+                                             (2, 288, 32, 16), (16, 24, 8, 16), (2, 450, 32, 16)])
 @pytest.mark.parametrize("mode", ["prompt", "decode", "pairs", "portions"])
 @pytest.mark.parametrize("cache_dtype,window", [(torch.float32, 37), (torch.bfloat16, 37), (torch.float32, 0), (torch.float32, 1)])
 def test_attention_over_a_shared_latent(H, rank, rot, page, mode, cache_dtype, window):

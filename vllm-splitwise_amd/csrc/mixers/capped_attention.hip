@@ -27,7 +27,7 @@ namespace swm {
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 
 constexpr int kQT = 32;               // query rows and keys per tile
-constexpr int kMaxBlocks = 12;        // 32-coordinate blocks of the larger of key and value size
+constexpr int kMaxBlocks = 16;        // 32-coordinate blocks of the larger of key and value size
 
 // N consecutive elements of a cache row as they are stored (bf16 two to a register), widened where they are used:
 // all loads of a key tile are issued before its first product, so their latencies overlap.
@@ -708,6 +708,10 @@ extern "C" int swm_masked_attention(void* out, const float* q, const void* key_c
     SWM_CAPPED_CASE(10)
     SWM_CAPPED_CASE(11)
     SWM_CAPPED_CASE(12)
+    SWM_CAPPED_CASE(13)
+    SWM_CAPPED_CASE(14)
+    SWM_CAPPED_CASE(15)
+    SWM_CAPPED_CASE(16)
   }
 #undef SWM_CAPPED_CASE
   return SW_OK;
