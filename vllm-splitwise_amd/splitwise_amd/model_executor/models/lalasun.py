@@ -187,6 +187,7 @@ class LalasunForCausalLM(nn.Module):
         self.norm = DynamicTanhNorm(cfg["width"])
         self.head = nn.Parameter(torch.zeros(cfg["vocab"], cfg["width"], dtype=dtype), requires_grad=False)
         self.sampler = Sampler(cfg["vocab"])
+        self.register_buffer("unit_weight", torch.ones(1, dtype=torch.float32), persistent=False)
         # set by a caller that wants the stream after every layer (a debugging aid; costs a copy per layer)
         self.keep_residuals: Optional[list] = None
 
@@ -224,12 +225,12 @@ class LalasunForCausalLM(nn.Module):
             raise RuntimeError("Lalasun steps need the ragged layout (InputMetadata.ragged)")
         positions = positions.reshape(-1)
         n = len(self.layers)
-        x0 = self.embed_tokens(input_ids)
-        # history[j]: X_j, the embedding rows and every layer's output before the depth mix; x: what the next layer reads
-        history = torch.empty(n + 1, x0.shape[0], x0.shape[1], dtype=torch.float32, device=x0.device)
-        history[0].copy_(x0)
-        x = history[0].clone()
-        h = (self.layers[0].norm1 if n else self.norm)(x, self.dtype)
+        x = self.embed_tokens(input_ids).float()
+        # history[j]: X_j, the embedding rows and every layer's output before the depth mix; x: what the next layer reads.
+        # The first launch files the embedding rows as entry 0 (a "mix" of that one entry) and takes the first norm.
+        history = torch.empty(n + 1, x.shape[0], x.shape[1], dtype=torch.float32, device=x.device)
+        h = (self.layers[0].norm1 if n else self.norm).gated_add_norm(x, self.dtype, history=history[:1],
+                                                                      depth_weights=self.unit_weight)
         for i, layer in enumerate(self.layers):
             y, gate = layer.mixer(h, positions, kv_caches[i], input_metadata)
             if layer.mlp is not None:
