@@ -64,12 +64,12 @@ def test_gated_stream_step(dtype, width):
             stream = x.clone().to(DEV)
             hd = hist.clone().to(DEV)
             out = torch.empty(rows, width, dtype=dtype, device=DEV) if use_norm else None
-            ops().gated_stream_step(stream, y.to(DEV) if use_y else None, gate.to(DEV) if use_gate else None, 0.7,
+            ops().gated_stream_step(stream, y.to(DEV) if use_y else None, gate.to(DEV) if use_gate else None, 0.6,
                                     hd[:n_hist] if use_hist else None, dw[:n_hist].contiguous().to(DEV) if use_hist else None,
                                     (alpha.to(DEV), w.to(DEV), b.to(DEV)) if use_norm else None, out)
             want = x.double()
             if use_y:
-                want = want + 0.7 * y.double() * (torch.sigmoid(gate.double()) if use_gate else 1.0)
+                want = want + 0.6 * y.double() * (torch.sigmoid(gate.double()) if use_gate else 1.0)
             if use_hist:
                 torch.testing.assert_close(hd[n_hist - 1].cpu().double(), want, atol=1e-5, rtol=1e-6)
                 torch.testing.assert_close(hd[n_hist:].cpu(), hist[n_hist:])              # later entries untouched
@@ -348,7 +348,7 @@ def _run_gla(proj, sizes, bias, tau, state, steps, H, d, dv):
     return outs
 
 
-@pytest.mark.parametrize("H,d,dv,tau,shift", [(3, 24, 16, 4.0, 1.0), (1, 8, 8, 16.0, 3.0), (2, 64, 48, 1.0, -2.0), (2, 100, 48, 0.25, -4.0),
+@pytest.mark.parametrize("H,d,dv,tau,shift", [(3, 24, 16, 4.0, 1.0), (1, 8, 8, 12.0, 3.0), (2, 64, 48, 1.0, -2.0), (2, 100, 48, 0.25, -4.0),
                                               (4, 40, 130, 2.0, 0.0), (1, 256, 64, 8.0, 2.0), (2, 32, 32, 0.05, -3.0)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gated_linear_attention_recurrence(H, d, dv, tau, shift, dtype):
@@ -391,7 +391,7 @@ def test_gated_linear_attention_recurrence(H, d, dv, tau, shift, dtype):
 # --------------------------------------------------------------- whole models through the engine
 def _cfg_a():
     layers = [lu.gla(2, 12, 20, 4.0), lu.latent(3, 8, 4, 12, 20, window=9), lu.attention(4, 2, 16, 8, chunk=11, rot_dims=8),
-              lu.latent(2, 16, 8, 8, 24, window=45, scale=0.2), lu.gla(3, 8, 8, 16.0), lu.attention(2, 2, 12, 12, chunk=32, rot_dims=12)]
+              lu.latent(2, 16, 8, 8, 24, window=45, scale=0.2), lu.gla(3, 8, 8, 12.0), lu.attention(2, 2, 12, 12, chunk=32, rot_dims=12)]
     mlps = [lu.dense(40), lu.dense(56), None, lu.dense(24), lu.dense(40), lu.dense(33)]
     return lu.config(layers, mlps, vocab=97, width=48, mult=0.8)
 

@@ -101,11 +101,11 @@ def _lalasun_preset(width: int, repeats: int, heads: int, kv_heads: int, ff: int
     latent-attention layers (a 192-wide latent plus 64 rotated coordinates per token, window 1024), an attention layer
     with grouped heads over chunks of 1024, and another gated-linear-attention layer, each with a dense feed-forward."""
     d = width // heads
-    gla = {"heads": heads, "dim": d // 2, "vdim": d, "tau": 16.0, "decay_rank": 16}
+    gla = {"heads": heads, "dim": d // 2, "vdim": d, "tau": 8.0, "decay_rank": 32}
     latent = {"heads": heads, "dim": d // 2, "rot_dim": 64, "vdim": d, "kv_rank": 192, "scale": (d // 2 + 64) ** -0.5,
-              "mask": {"size": 1024}, "rot": {"base": 1000000.0, "dims": 64}}
+              "mask": {"size": 1024}, "rot": {"base": 10000.0, "dims": 64}}
     attn = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024},
-            "rot": {"base": 500000.0, "dims": d}}
+            "rot": {"base": 100000.0, "dims": d}}
     dense = {"kind": "dense", "ff": ff}
     layers = []
     for _ in range(repeats):

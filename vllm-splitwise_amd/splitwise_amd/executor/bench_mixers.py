@@ -486,7 +486,7 @@ def kernel_table_lalasun(width: int = 2048, heads: int = 16, kv_heads: int = 4, 
         state = torch.zeros(max(B, 2), heads, dk, d, device=dev)
         go = torch.empty(T, heads * d, device=dev)
         t = _time(lambda: _C.mixer_ops.gla(go, gproj[:, :heads * dk], gproj[:, heads * dk:2 * heads * dk],
-                                           gproj[:, 2 * heads * dk:], zpre, zbias, 16.0, dk ** -0.5, state, lbatch, heads, dk, d))
+                                           gproj[:, 2 * heads * dk:], zpre, zbias, 8.0, dk ** -0.5, state, lbatch, heads, dk, d))
         chunk = 32
         gflops = T * heads * (2.0 * chunk * dk + 2.0 * chunk * d + 4.0 * dk * d)
         gbytes = T * heads * ((3 * dk + d) * 2 + d * 4) + 2 * B * heads * dk * d * 4
