@@ -6,8 +6,10 @@
  * attention over a sliding window plus kept first tokens with the heads' weights mixed after the
  * softmax, norms with a single gain; linear attention with a decay per head, soft-capped gated attention
  * with partial rotary embedding, routed experts with group-limited choice, and the fused residual-add + norm
- * of layers whose sublayers run side by side.  A library of its own so that a model that needs only
- * these compiles only these.
+ * of layers whose sublayers run side by side; attention over chunks with an extra softmax term and over a
+ * latent shared by all heads, gated linear attention with a decay per key channel, and the gated residual
+ * step of layers that read a mix of all earlier layers' outputs.  A library of its own so that a model that
+ * needs only these compiles only these.
  *
  * A step is a RAGGED batch: the new tokens of all sequences back to back in one token dimension.
  *   q_start[B + 1]   first row of every sequence's tokens (int32, ascending, q_start[B] = rows)
