@@ -8,8 +8,10 @@
  * with partial rotary embedding, routed experts with group-limited choice, and the fused residual-add + norm
  * of layers whose sublayers run side by side; attention over chunks with an extra softmax term and over a
  * latent shared by all heads, gated linear attention with a decay per key channel, and the gated residual
- * step of layers that read a mix of all earlier layers' outputs.  A library of its own so that a model that
- * needs only these compiles only these.
+ * step of layers that read a mix of all earlier layers' outputs; norms in groups of channels around every
+ * sublayer, a causal convolution added to a sublayer's input, the delta rule with one decay per head, attention
+ * with sigmoid weights and a softmax router.  A library of its own so that a model that needs only these compiles
+ * only these.
  *
  * A step is a RAGGED batch: the new tokens of all sequences back to back in one token dimension.
  *   q_start[B + 1]   first row of every sequence's tokens (int32, ascending, q_start[B] = rows)
@@ -34,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SWM_ABI_VERSION 3
+#define SWM_ABI_VERSION 4
 int swm_abi_version(void);
 const char* swm_last_error(void);
 
@@ -136,6 +138,7 @@ int swm_expert_down(float* out, const void* hidden, const void* down, const int3
  * (pair_weight fp32 [rows * top], NULL: all 1). */
 #define SWM_ACT_GELU 0
 #define SWM_ACT_RELU2 1
+#define SWM_ACT_NONE 2 /* the products as they are: the hidden layer's gated unit is a kernel of its own */
 int swm_expert_up(void* hidden, const void* x, const void* up, const int32_t* order, const int32_t* expert_start,
                   int num_experts, int64_t sorted_rows, int width, int ff, int top, int activation, int act_dtype,
                   void* stream);
@@ -275,6 +278,57 @@ int swm_lightning(float* out, const void* q, const void* k, const void* v, int64
                   float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows,
                   int num_seqs, int max_query_len, int heads, int dim, int vdim, float* workspace, int act_dtype,
                   void* stream);
+
+/* ---- layers with a norm before AND after each sublayer, taken in groups of channels ---- */
+
+/* N(u; w): the row cut into `groups` equal runs of channels, each run divided by its own sqrt(mean(run^2) + eps),
+ * the row times w (fp32 [width]).  With y1:  residual[t] += layer_scale * N(s1 * y1[t] + s2 * y2[t]; post_w)
+ * (y2 NULL: one addend; layer_scale fp32 [width] or NULL; y1, y2 of y_dtype with row strides).  With out:
+ * out[t] = out_dtype(N(residual[t]; w)) of the new residual.  residual fp32 [rows, width]. */
+int swm_group_norm_add(float* residual, const void* y1, int64_t y1_stride, float s1, const void* y2,
+                       int64_t y2_stride, float s2, int y_dtype, const float* post_w, const float* layer_scale,
+                       const float* w, void* out, int out_dtype, int groups, float eps, int64_t rows, int width,
+                       void* stream);
+
+/* The short causal convolution of swm_short_conv with the types and the form named: x of x_dtype, out of out_dtype
+ * [rows, channels]; out = act(conv(x) + (residual != 0 ? x : 0)), act = silu when silu != 0.  The state holds the last
+ * num_taps - 1 inputs in fp32; swm_short_conv_advance (with x's dtype) moves it on. */
+int swm_causal_conv(void* out, int out_dtype, const void* x, int x_dtype, int64_t x_stride, const float* taps,
+                    const float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
+                    const int32_t* state_slot, int64_t rows, int channels, int num_taps, int silu, int residual,
+                    void* stream);
+
+/* swm_channel_delta with ONE decay per head: g = exp(-exp(a_log[head]) * softplus(decay_pre[t, head] + dt_bias[head])),
+ * decay_pre act_dtype [rows, heads] (row stride decay_stride), dt_bias fp32 [heads].  Workspace as swm_channel_delta. */
+int swm_gated_delta(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride, const void* decay_pre,
+                    int64_t decay_stride, const float* dt_bias, const float* a_log, float* state,
+                    const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows,
+                    int num_seqs, int heads, int kv_heads, int dim, int vdim, float* workspace, int act_dtype,
+                    void* stream);
+
+/* swm_rope_cache behind an RMS norm of every query and key head over its `dim` coordinates:
+ * x / sqrt(mean(x^2) + norm_eps) * q_norm (k_norm), fp32 [dim] weights shared by the heads; q_norm NULL: no norm. */
+int swm_norm_rope_cache(float* q_out, const void* q, const void* k, const void* v, int64_t in_stride,
+                        const float* q_norm, const float* k_norm, float norm_eps, const int64_t* positions,
+                        const float* inv_freq, int rot_dims, int pair_halves, void* key_cache, void* value_cache,
+                        const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim, int vdim,
+                        int act_dtype, void* stream);
+
+/* Attention WITHOUT a softmax over the layout of swm_masked_attention: a key that position i sees (j <= i, and
+ * i - j < window when window > 0) weighs sigmoid((q . k) * scale + score_bias[head]) (score_bias fp32 [heads]); the
+ * weights are not normalised over the keys.  Gate, caches, workspace (swm_masked_attention_workspace_floats) as there. */
+int swm_sigmoid_attention(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
+                          int64_t gate_stride, const float* score_bias, const int32_t* block_tables, int table_width,
+                          const int32_t* q_start, const int32_t* ctx_len, int64_t rows, int num_seqs,
+                          int max_query_len, int heads, int kv_heads, int dim, int vdim, int page_size, float scale,
+                          int window, float* workspace, int act_dtype, void* stream);
+
+/* swm_group_router with the scores, the groups' scores and the weights named: softmax != 0: s = softmax(logits) over
+ * all experts (else sigmoid); group_best_one != 0: a group scores its largest choice score (else the sum of its two
+ * largest); normalize == 0: weights = s of the chosen * scale, not divided by their sum. */
+int swm_group_router_as(int32_t* chosen, float* weights, const float* logits, const float* correction, int64_t rows,
+                        int experts, int top, int groups, int keep, float scale, int softmax, int group_best_one,
+                        int normalize, void* stream);
 
 #ifdef __cplusplus
 }

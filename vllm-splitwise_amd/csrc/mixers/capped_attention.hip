@@ -116,8 +116,9 @@ __global__ __launch_bounds__(64 * max_waves_of(NB)) void capped_attention_kernel
     const void* __restrict__ value_cache, const void* __restrict__ gate, int64_t gate_stride,
     const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
-    float scale, float softcap, int window, int chunk, int sink, int64_t k_stride, int64_t v_stride, int tpt, int split,
-    int rows_used, int page_shift, float* __restrict__ partial, int64_t total_rows) {
+    float scale, float softcap, int window, int chunk, int sink, const float* __restrict__ score_bias, int64_t k_stride,
+    int64_t v_stride, int tpt, int split, int rows_used, int page_shift, float* __restrict__ partial,
+    int64_t total_rows) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int R = heads / kv_heads;
   const int dblocks = (dim + 31) / 32;
@@ -163,6 +164,10 @@ __global__ __launch_bounds__(64 * max_waves_of(NB)) void capped_attention_kernel
   const int tile_lo = lowest / kQT, tile_hi = live ? last_pos / kQT : -1;
   const bool kvec = dim % 8 == 0 && k_stride % 8 == 0;
   const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
+  // score_bias: a seen key weighs sigmoid(score + bias of the query's head) and nothing is normalised over the keys;
+  // the running maximum then stays 0 (every part's factor is 1) and the denominator is never used
+  const bool sig = score_bias != nullptr;
+  const float bias_q = sig ? score_bias[g * R + qi % R] : 0.0f;
 
   f32x16 o[NVB];
 #pragma unroll
@@ -242,29 +247,40 @@ __global__ __launch_bounds__(64 * max_waves_of(NB)) void capped_attention_kernel
       float v = s[r];
       if (softcap > 0.0f) v = softcap * fast_tanhf_(v * inv_cap);
       const bool seen = kj <= pos_q && kj >= low_q;
-      v = seen ? v : -INFINITY;
-      p[r] = v;
-      tmax = fmaxf(tmax, v);
+      if (sig) {
+        p[r] = seen ? __builtin_amdgcn_rcpf(1.0f + fast_expf_(-(v + bias_q))) : 0.0f;
+      } else {
+        v = seen ? v : -INFINITY;
+        p[r] = v;
+        tmax = fmaxf(tmax, v);
+      }
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m_run, tmax);
-    const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-    const float alpha = fast_expf_(m_run - m_use);           // 0 while nothing has been seen
-    float psum = 0.0f;
+    float alpha = 1.0f;
+    if (sig) {
+      m_run = 0.0f;
+    } else {
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run, tmax);
+      const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+      alpha = fast_expf_(m_run - m_use);                     // 0 while nothing has been seen
+      float psum = 0.0f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      p[r] = fast_expf_(p[r] - m_use);
-      psum += p[r];
+      for (int r = 0; r < 16; ++r) {
+        p[r] = fast_expf_(p[r] - m_use);
+        psum += p[r];
+      }
+      psum += __shfl_xor(psum, 32, 64);
+      l_run = l_run * alpha + psum;
+      m_run = m_new;
     }
-    psum += __shfl_xor(psum, 32, 64);
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
     // ---- O^T = alpha O^T + V^T P^T
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
       if (b < vdim) {                                          // block b holds the channels NB * lane + b
+        if (!sig) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+          for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+        }
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vraw[r].get(b), p[r], o[b], 0, 0, 0);
       }
@@ -329,7 +345,7 @@ __global__ __launch_bounds__(64 * max_waves_of(NB)) void capped_attention_kernel
         den += f * Ml[(w * kQT + r) * 2 + 1];
         num += f * Oall[(w * rows_used + r) * ostride + c];
       }
-      float v = num / den;
+      float v = sig ? num : num / den;
       const int64_t col = (int64_t)(g * R + hh) * vdim + c;
       if (gate != nullptr) v *= sigmoidf_(ld<T>(gate, (row0 + tt) * gate_stride + col));
       st<T>(out, (row0 + tt) * (int64_t)heads * vdim + col, v);
@@ -341,7 +357,7 @@ __global__ __launch_bounds__(64 * max_waves_of(NB)) void capped_attention_kernel
   if (live) {
     const float m_fin = sink ? fmaxf(m_run, 0.0f) : m_run;
     const float fin = sink ? expf(m_run - m_fin) : 1.0f;
-    const float inv = fin / (l_run * fin + (sink ? expf(-m_fin) : 0.0f));
+    const float inv = sig ? 1.0f : fin / (l_run * fin + (sink ? expf(-m_fin) : 0.0f));
 #pragma unroll
     for (int b = 0; b < NVB; ++b)
 #pragma unroll
@@ -371,9 +387,11 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
     const void* __restrict__ value_cache, const void* __restrict__ gate, int64_t gate_stride,
     const int32_t* __restrict__ block_tables, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, int heads, int kv_heads, int dim, int vdim, int page_size, int page_shift,
-    float scale, float softcap, int window, int chunk, int sink, int64_t k_stride, int64_t v_stride) {
+    float scale, float softcap, int window, int chunk, int sink, const float* __restrict__ score_bias, int64_t k_stride,
+    int64_t v_stride) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int seq = blockIdx.x, g = blockIdx.y, R = heads / kv_heads;
+  const bool sig = score_bias != nullptr;                    // sigmoid weights: see capped_attention_kernel
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, pt = lane % LK, grp = lane / LK, nw = blockDim.x >> 6;
   const int row0 = q_start[seq], n = q_start[seq + 1] - row0;
   if (n <= 0) return;                                        // the whole workgroup
@@ -382,11 +400,12 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
   float* Ml = lds;                                           // [nw][RQ][2]
   float* Os = lds + nw * RQ * 2;                             // [nw][RQ][LK * C]
 
-  float qv[RQ][C], o[RQ][C], m_run[RQ], l_run[RQ];
+  float qv[RQ][C], o[RQ][C], m_run[RQ], l_run[RQ], bias[RQ];
   int pos[RQ], low[RQ];
 #pragma unroll
   for (int r = 0; r < RQ; ++r) {
     const int tt = r / R, hh = r % R;
+    bias[r] = sig ? score_bias[g * R + hh] : 0.0f;
     pos[r] = ctx + min(tt, n - 1);                           // padding rows behave like the last token's
     low[r] = chunk > 0 ? pos[r] / chunk * chunk : window > 0 ? pos[r] - window + 1 : 0;
     m_run[r] = -INFINITY;
@@ -429,6 +448,13 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
         s = lanes_sum<LK>(s);
         if (softcap > 0.0f) s = softcap * fast_tanhf_(s * inv_cap);
         const bool seen = key <= pos[r] && key >= low[r];
+        if (sig) {
+          const float p = seen ? __builtin_amdgcn_rcpf(1.0f + fast_expf_(-(s + bias[r]))) : 0.0f;
+          m_run[r] = 0.0f;
+#pragma unroll
+          for (int c = 0; c < C; ++c) o[r][c] += p * vr[u].get(c);
+          continue;
+        }
         if (!seen) s = -INFINITY;
         const float m_new = fmaxf(m_run[r], s);
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
@@ -481,7 +507,7 @@ __global__ __launch_bounds__(512) void capped_attention_rows_kernel(
       den += f * Ml[(w * RQ + r) * 2 + 1];
       num += f * Os[(w * RQ + r) * LK * C + c];
     }
-    float v = num / den;
+    float v = sig ? num : num / den;
     const int64_t col = (int64_t)(g * R + hh) * vdim + c;
     if (gate != nullptr) v *= sigmoidf_(ld<T>(gate, (row0 + tt) * gate_stride + col));
     st<T>(out, (int64_t)(row0 + tt) * heads * vdim + col, v);
@@ -492,8 +518,8 @@ template <typename T, int RQ, int C, int LK>
 int launch_capped_rows(void* out, const float* q, const void* key_cache, const void* value_cache, const void* gate,
                        int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
                        const int32_t* ctx_len, int num_seqs, int heads, int kv_heads, int dim, int vdim, int page_size,
-                       float scale, float softcap, int window, int chunk, int sink, int64_t k_stride, int64_t v_stride,
-                       hipStream_t stream) {
+                       float scale, float softcap, int window, int chunk, int sink, const float* score_bias, int64_t k_stride,
+                       int64_t v_stride, hipStream_t stream) {
   constexpr bool half = sizeof(typename Conv<T>::store_t) == 2;
   constexpr int U = RQ * C <= 32 ? (half ? 4 : 2) : (half ? 2 : 1);
   const int nw = 8;
@@ -510,7 +536,8 @@ int launch_capped_rows(void* out, const float* q, const void* key_cache, const v
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)num_seqs, (unsigned)kv_heads), dim3(64 * nw), lds_bytes, stream, out, q,
                      key_cache, value_cache, gate, gate_stride, block_tables, table_width, q_start, ctx_len, heads,
-                     kv_heads, dim, vdim, page_size, page_shift, scale, softcap, window, chunk, sink, k_stride, v_stride);
+                     kv_heads, dim, vdim, page_size, page_shift, scale, softcap, window, chunk, sink, score_bias, k_stride,
+                     v_stride);
   SW_CHECK_LAUNCH();
   return SW_OK;
 }
@@ -521,7 +548,7 @@ bool try_capped_rows(int* status, int rows_used, void* out, const float* q, cons
                      const void* value_cache, const void* gate, int64_t gate_stride, const int32_t* block_tables,
                      int table_width, const int32_t* q_start, const int32_t* ctx_len, int num_seqs, int heads,
                      int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window, int chunk,
-                     int sink, int64_t k_stride, int64_t v_stride, hipStream_t stream) {
+                     int sink, const float* score_bias, int64_t k_stride, int64_t v_stride, hipStream_t stream) {
   if (rows_used > 8) return false;
   auto pow2 = [](int x) { return x <= 4 ? 4 : x <= 8 ? 8 : x <= 16 ? 16 : x <= 32 ? 32 : 64; };
   const int most = std::max(dim, vdim);
@@ -537,8 +564,8 @@ bool try_capped_rows(int* status, int rows_used, void* out, const float* q, cons
   if (rq == RQV && c == CV && lk == LKV) {                                                                              \
     *status = launch_capped_rows<T, RQV, CV, LKV>(out, q, key_cache, value_cache, gate, gate_stride, block_tables,      \
                                                   table_width, q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim,  \
-                                                  page_size, scale, softcap, window, chunk, sink, k_stride, v_stride,   \
-                                                  stream);                                                              \
+                                                  page_size, scale, softcap, window, chunk, sink, score_bias, k_stride, \
+                                                  v_stride, stream);                                                              \
     return true;                                                                                                        \
   }
   SWM_ROWS_CASE(1, 4, 8) SWM_ROWS_CASE(1, 8, 8) SWM_ROWS_CASE(1, 16, 8) SWM_ROWS_CASE(1, 32, 8)
@@ -555,7 +582,7 @@ bool try_capped_rows(int* status, int rows_used, void* out, const float* q, cons
 template <typename T>
 __global__ __launch_bounds__(256) void capped_attention_join_kernel(
     void* __restrict__ out, const float* __restrict__ partial, const void* __restrict__ gate, int64_t gate_stride,
-    int64_t total_rows, int heads, int vdim, int parts, int sink) {
+    int64_t total_rows, int heads, int vdim, int parts, int sink, int sig) {
   const int64_t rh = blockIdx.x;                             // row * heads + head
   const float* ml = partial;
   const float* po = partial + (int64_t)parts * total_rows * heads * 2;
@@ -575,7 +602,7 @@ __global__ __launch_bounds__(256) void capped_attention_join_kernel(
       const float m = ml[(z * part_stride + rh) * 2];
       if (m != -INFINITY) num += expf(m - m_all) * po[(z * part_stride + rh) * vdim + c];
     }
-    float v = num / den;
+    float v = sig ? num : num / den;
     if (gate != nullptr) v *= sigmoidf_(ld<T>(gate, t * gate_stride + (int64_t)hd * vdim + c));
     st<T>(out, rh * vdim + c, v);
   }
@@ -602,8 +629,8 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
                             int64_t gate_stride, const int32_t* block_tables, int table_width, const int32_t* q_start,
                             const int32_t* ctx_len, int64_t rows, int num_seqs, int max_query_len, int heads,
                             int kv_heads, int dim, int vdim, int page_size, float scale, float softcap, int window,
-                            int chunk, int sink, int64_t k_stride, int64_t v_stride, float* workspace,
-                            hipStream_t stream) {
+                            int chunk, int sink, const float* score_bias, int64_t k_stride, int64_t v_stride,
+                            float* workspace, hipStream_t stream) {
   const int R = heads / kv_heads;
   const int tpt = kQT / R;
   const int qstride = (dim + 31) / 32 * 32 + 4, ostride = NB * 32 + 1;
@@ -613,7 +640,7 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
     int status = SW_OK;
     if (try_capped_rows<T>(&status, rows_used, out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width,
                            q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim, page_size, scale, softcap, window,
-                           chunk, sink, k_stride, v_stride, stream))
+                           chunk, sink, score_bias, k_stride, v_stride, stream))
       return status;
   }
   auto lds_bytes = [&](int nw) {
@@ -644,12 +671,12 @@ int launch_capped_attention(void* out, const float* q, const void* key_cache, co
   const dim3 grid((unsigned)(split ? tiles : (tiles + nw - 1) / nw), (unsigned)kv_heads, (unsigned)parts);
   hipLaunchKernelGGL(kernel, grid, dim3(64 * nw), lds_bytes(nw), stream, out, q, key_cache, value_cache, gate,
                      gate_stride, block_tables, table_width, q_start, ctx_len, num_seqs, heads, kv_heads, dim, vdim,
-                     page_size, scale, softcap, window, chunk, sink, k_stride, v_stride, tpt, split ? 1 : 0, rows_used,
-                     page_shift, parts > 1 ? workspace : (float*)nullptr, rows);
+                     page_size, scale, softcap, window, chunk, sink, score_bias, k_stride, v_stride, tpt, split ? 1 : 0,
+                     rows_used, page_shift, parts > 1 ? workspace : (float*)nullptr, rows);
   SW_CHECK_LAUNCH();
   if (parts > 1) {
     hipLaunchKernelGGL(capped_attention_join_kernel<T>, dim3((unsigned)(rows * heads)), dim3(vdim <= 64 ? 64 : 128), 0,
-                       stream, out, workspace, gate, gate_stride, rows, heads, vdim, parts, sink);
+                       stream, out, workspace, gate, gate_stride, rows, heads, vdim, parts, sink, score_bias != nullptr ? 1 : 0);
     SW_CHECK_LAUNCH();
   }
   return SW_OK;
@@ -665,12 +692,12 @@ extern "C" int64_t swm_masked_attention_workspace_floats(int64_t rows, int num_s
   return parts > 1 ? (int64_t)parts * rows * heads * (vdim + 2) : 0;
 }
 
-extern "C" int swm_masked_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
-                                    const void* gate, int64_t gate_stride, const int32_t* block_tables,
-                                    int table_width, const int32_t* q_start, const int32_t* ctx_len, int64_t rows,
-                                    int num_seqs, int max_query_len, int heads, int kv_heads, int dim, int vdim,
-                                    int page_size, float scale, float softcap, int window, int chunk, int sink,
-                                    int64_t k_stride, int64_t v_stride, float* workspace, int act_dtype, void* stream) {
+static int masked_attention_impl(void* out, const float* q, const void* key_cache, const void* value_cache,
+                                 const void* gate, int64_t gate_stride, const int32_t* block_tables, int table_width,
+                                 const int32_t* q_start, const int32_t* ctx_len, int64_t rows, int num_seqs,
+                                 int max_query_len, int heads, int kv_heads, int dim, int vdim, int page_size,
+                                 float scale, float softcap, int window, int chunk, int sink, const float* score_bias,
+                                 int64_t k_stride, int64_t v_stride, float* workspace, int act_dtype, void* stream) {
   using namespace swm;
   if (rows == 0 || num_seqs == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "masked_attention: unsupported dtype %d", act_dtype);
@@ -692,8 +719,8 @@ extern "C" int swm_masked_attention(void* out, const float* q, const void* key_c
     SWM_DISPATCH_ACT(act_dtype, return (launch_capped_attention<T, N>(                                                  \
                                     out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width,       \
                                     q_start, ctx_len, rows, num_seqs, max_query_len, heads, kv_heads, dim, vdim,        \
-                                    page_size, scale, softcap, window, chunk, sink, k_stride, v_stride, workspace,      \
-                                    s)););                                                                              \
+                                    page_size, scale, softcap, window, chunk, sink, score_bias, k_stride, v_stride,     \
+                                    workspace, s)););                                                                              \
     break;
   switch (nvb) {
     SWM_CAPPED_CASE(1)
@@ -715,6 +742,33 @@ extern "C" int swm_masked_attention(void* out, const float* q, const void* key_c
   }
 #undef SWM_CAPPED_CASE
   return SW_OK;
+}
+
+extern "C" int swm_masked_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
+                                    const void* gate, int64_t gate_stride, const int32_t* block_tables,
+                                    int table_width, const int32_t* q_start, const int32_t* ctx_len, int64_t rows,
+                                    int num_seqs, int max_query_len, int heads, int kv_heads, int dim, int vdim,
+                                    int page_size, float scale, float softcap, int window, int chunk, int sink,
+                                    int64_t k_stride, int64_t v_stride, float* workspace, int act_dtype, void* stream) {
+  return masked_attention_impl(out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width, q_start,
+                               ctx_len, rows, num_seqs, max_query_len, heads, kv_heads, dim, vdim, page_size, scale,
+                               softcap, window, chunk, sink, nullptr, k_stride, v_stride, workspace, act_dtype, stream);
+}
+
+extern "C" int swm_sigmoid_attention(void* out, const float* q, const void* key_cache, const void* value_cache,
+                                     const void* gate, int64_t gate_stride, const float* score_bias,
+                                     const int32_t* block_tables, int table_width, const int32_t* q_start,
+                                     const int32_t* ctx_len, int64_t rows, int num_seqs, int max_query_len, int heads,
+                                     int kv_heads, int dim, int vdim, int page_size, float scale, int window,
+                                     float* workspace, int act_dtype, void* stream) {
+  if (score_bias == nullptr) {
+    sw::set_error("sigmoid_attention: the per-head bias is missing (a layer without one passes zeros)");
+    return SW_ERR_INVALID;
+  }
+  return masked_attention_impl(out, q, key_cache, value_cache, gate, gate_stride, block_tables, table_width, q_start,
+                               ctx_len, rows, num_seqs, max_query_len, heads, kv_heads, dim, vdim, page_size, scale,
+                               0.0f, window, 0, 0, score_bias, (int64_t)kv_heads * dim, (int64_t)kv_heads * vdim,
+                               workspace, act_dtype, stream);
 }
 
 extern "C" int swm_capped_attention(void* out, const float* q, const void* key_cache, const void* value_cache,

@@ -40,8 +40,9 @@ __device__ __forceinline__ float group_sum(float v) {
 template <typename T>
 __global__ __launch_bounds__(kPrepThreads) void channel_delta_prep_kernel(
     float* __restrict__ ops, float* __restrict__ beta, const float* __restrict__ qkv,
-    const void* __restrict__ beta_pre, int64_t beta_stride, const void* __restrict__ decay_pre,
-    const float* __restrict__ dt_bias, const float* __restrict__ a_log, int heads, int kv_heads, int dim, int vdim) {
+    const void* __restrict__ beta_pre, int64_t beta_stride, const void* __restrict__ decay_pre, int64_t decay_stride,
+    int decay_per_head, const float* __restrict__ dt_bias, const float* __restrict__ a_log, int heads, int kv_heads,
+    int dim, int vdim) {
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t row_w = 2 * (int64_t)kv_heads * dim + (int64_t)heads * vdim;
@@ -61,14 +62,19 @@ __global__ __launch_bounds__(kPrepThreads) void channel_delta_prep_kernel(
     kk = sw::wave_sum(kk);
     const float qf = qscale / sqrtf(qq + 1e-6f), kf = 1.0f / sqrtf(kk + 1e-6f);
     const float rate = expf(a_log[h]);
+    // one decay for the whole head (every key channel gets the same number), or one per key channel
+    const float head_decay =
+        decay_per_head ? expf(-rate * softplusf_(ld<T>(decay_pre, t * decay_stride + h) + dt_bias[h])) : 0.0f;
     const int dimp = (dim + 3) & ~3;                     // operand rows are padded to whole 16-byte pieces
     float* o = ops + (t * heads + h) * 3 * (int64_t)dimp;
     for (int i = lane; i < dimp; i += 64) {
       const bool in = i < dim;
       o[i] = in ? q[i] * qf : 0.0f;
       o[dimp + i] = in ? k[i] * kf : 0.0f;
-      o[2 * dimp + i] = in ? expf(-rate * softplusf_(ld<T>(decay_pre, (t * heads + h) * (int64_t)dim + i) + dt_bias[h * dim + i]))
-                           : 0.0f;
+      float gdec = head_decay;
+      if (in && !decay_per_head)
+        gdec = expf(-rate * softplusf_(ld<T>(decay_pre, t * decay_stride + (int64_t)h * dim + i) + dt_bias[h * dim + i]));
+      o[2 * dimp + i] = in ? gdec : 0.0f;
     }
     if (lane == 0) beta[t * heads + h] = sigmoidf_(ld<T>(beta_pre, t * beta_stride + h));
   }
@@ -303,11 +309,11 @@ int64_t swm_general_delta_workspace_floats(int64_t rows, int heads, int dim) {
   return rows * heads * 4 * (int64_t)((dim + 3) & ~3);
 }
 
-int swm_channel_delta(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride,
-                      const void* decay_pre, const float* dt_bias, const float* a_log, float* state,
-                      const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows,
-                      int num_seqs, int heads, int kv_heads, int dim, int vdim, float* workspace, int act_dtype,
-                      void* stream) {
+static int delta_with_decay(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride,
+                            const void* decay_pre, int64_t decay_stride, int decay_per_head, const float* dt_bias,
+                            const float* a_log, float* state, const int32_t* q_start, const int32_t* ctx_len,
+                            const int32_t* state_slot, int64_t rows, int num_seqs, int heads, int kv_heads, int dim,
+                            int vdim, float* workspace, int act_dtype, void* stream) {
   using namespace swm;
   if (num_seqs == 0 || rows == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "channel_delta: unsupported dtype %d", act_dtype);
@@ -319,8 +325,8 @@ int swm_channel_delta(float* out, const float* qkv, const void* beta_pre, int64_
   float* ops = workspace;
   float* beta = workspace + rows * heads * 3 * (int64_t)((dim + 3) & ~3);
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(channel_delta_prep_kernel<T>, dim3((unsigned)rows), dim3(kPrepThreads), 0,
-                                                 s, ops, beta, qkv, beta_pre, beta_stride, decay_pre, dt_bias, a_log,
-                                                 heads, kv_heads, dim, vdim););
+                                                 s, ops, beta, qkv, beta_pre, beta_stride, decay_pre, decay_stride,
+                                                 decay_per_head, dt_bias, a_log, heads, kv_heads, dim, vdim););
   SW_CHECK_LAUNCH();
   const dim3 grid((unsigned)((vdim + kColsPerWave - 1) / kColsPerWave), (unsigned)heads, (unsigned)num_seqs);
   const int64_t row_w = 2 * (int64_t)kv_heads * dim + (int64_t)heads * vdim;
@@ -331,6 +337,25 @@ int swm_channel_delta(float* out, const float* qkv, const void* beta_pre, int64_
                                             vdim););
   SW_CHECK_LAUNCH();
   return SW_OK;
+}
+
+int swm_channel_delta(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride,
+                      const void* decay_pre, const float* dt_bias, const float* a_log, float* state,
+                      const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows,
+                      int num_seqs, int heads, int kv_heads, int dim, int vdim, float* workspace, int act_dtype,
+                      void* stream) {
+  return delta_with_decay(out, qkv, beta_pre, beta_stride, decay_pre, (int64_t)heads * dim, 0, dt_bias, a_log, state,
+                          q_start, ctx_len, state_slot, rows, num_seqs, heads, kv_heads, dim, vdim, workspace, act_dtype,
+                          stream);
+}
+
+int swm_gated_delta(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride, const void* decay_pre,
+                    int64_t decay_stride, const float* dt_bias, const float* a_log, float* state,
+                    const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot, int64_t rows,
+                    int num_seqs, int heads, int kv_heads, int dim, int vdim, float* workspace, int act_dtype,
+                    void* stream) {
+  return delta_with_decay(out, qkv, beta_pre, beta_stride, decay_pre, decay_stride, 1, dt_bias, a_log, state, q_start,
+                          ctx_len, state_slot, rows, num_seqs, heads, kv_heads, dim, vdim, workspace, act_dtype, stream);
 }
 
 int swm_general_delta(float* out, const void* r, const void* k, const void* v, int64_t rkv_stride,

@@ -13,8 +13,10 @@ namespace swm {
 constexpr int TM = 32, TN = 64, TK = 32, kFfnThreads = 256;
 
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
-// activation of an expert's hidden layer: SWM_ACT_GELU (exact gelu) or SWM_ACT_RELU2 (the square of relu)
+// activation of an expert's hidden layer: SWM_ACT_GELU (exact gelu), SWM_ACT_RELU2 (the square of relu) or
+// SWM_ACT_NONE (the products as they are, for a gated unit that a kernel of its own applies)
 __device__ __forceinline__ float expert_act(float z, int activation) {
+  if (activation == SWM_ACT_NONE) return z;
   if (activation == SWM_ACT_RELU2) {
     const float r = fmaxf(z, 0.0f);
     return r * r;
@@ -247,7 +249,8 @@ int swm_expert_up(void* hidden, const void* x, const void* up, const int32_t* or
                   void* stream) {
   using namespace swm;
   if (sorted_rows == 0) return SW_OK;
-  SW_CHECK_ARG(activation == SWM_ACT_GELU || activation == SWM_ACT_RELU2, "expert_up: unknown activation %d", activation);
+  SW_CHECK_ARG(activation == SWM_ACT_GELU || activation == SWM_ACT_RELU2 || activation == SWM_ACT_NONE,
+               "expert_up: unknown activation %d", activation);
   SW_CHECK_ARG(act_ok(act_dtype), "expert_up_gelu: unsupported dtype %d", act_dtype);
   SW_CHECK_ARG(num_experts > 0 && width > 0 && ff > 0 && top > 0 && sorted_rows < (1ll << 30), "expert_up_gelu: bad shape");
   if (act_dtype == SW_BF16 && width % 8 == 0) {

@@ -120,11 +120,14 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(
 // ------------------------------------------------------------------------- short convolution + silu
 constexpr int kMaxTaps = 16;
 
-template <typename T>
+// TX: type of the inputs x, TO: type of the outputs.  silu: the activation after the sum; residual: the input
+// itself is added to its convolution (out = x + conv(x)).
+template <typename TX, typename TO>
 __global__ __launch_bounds__(kRowThreads) void short_conv_kernel(
-    float* __restrict__ out, const void* __restrict__ x, int64_t x_stride, const float* __restrict__ taps,
+    void* __restrict__ out, const void* __restrict__ x, int64_t x_stride, const float* __restrict__ taps,
     const float* __restrict__ state, const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
-    const int32_t* __restrict__ token_seq, const int32_t* __restrict__ state_slot, int channels, int num_taps) {
+    const int32_t* __restrict__ token_seq, const int32_t* __restrict__ state_slot, int channels, int num_taps, int silu,
+    int residual) {
   const int64_t t = blockIdx.x;
   const int c = blockIdx.y * kRowThreads + threadIdx.x;
   if (c >= channels) return;
@@ -138,7 +141,7 @@ __global__ __launch_bounds__(kRowThreads) void short_conv_kernel(
     const int64_t src = t - back;
     float xv;
     if (src >= first) {
-      xv = ld<T>(x, src * x_stride + c);
+      xv = ld<TX>(x, src * x_stride + c);
     } else if (carried) {
       // the input `first - src` tokens before this step's first one: the state's row (num_taps-1) - that
       xv = carry[(int64_t)(num_taps - 1 - (first - (int)src)) * channels + c];
@@ -147,7 +150,8 @@ __global__ __launch_bounds__(kRowThreads) void short_conv_kernel(
     }
     acc += taps[(int64_t)c * num_taps + j] * xv;
   }
-  out[t * (int64_t)channels + c] = acc * sigmoidf_(acc);
+  if (residual) acc += ld<TX>(x, t * x_stride + c);
+  st<TO>(out, t * (int64_t)channels + c, silu ? acc * sigmoidf_(acc) : acc);
 }
 
 // one thread per (sequence, channel): reads what it needs of the old state, then writes the new one
@@ -259,15 +263,30 @@ int swm_short_conv(float* out, const void* x, int64_t x_stride, const float* tap
                    const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
                    const int32_t* state_slot, int64_t rows, int channels, int num_taps, int act_dtype,
                    void* stream) {
+  return swm_causal_conv(out, SW_F32, x, act_dtype, x_stride, taps, state, q_start, ctx_len, token_seq, state_slot, rows,
+                         channels, num_taps, 1, 0, stream);
+}
+
+int swm_causal_conv(void* out, int out_dtype, const void* x, int x_dtype, int64_t x_stride, const float* taps,
+                    const float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
+                    const int32_t* state_slot, int64_t rows, int channels, int num_taps, int silu, int residual,
+                    void* stream) {
   using namespace swm;
   if (rows == 0) return SW_OK;
-  SW_CHECK_ARG(act_ok(act_dtype), "short_conv: unsupported dtype %d", act_dtype);
+  SW_CHECK_ARG(act_ok(x_dtype) && act_ok(out_dtype), "causal_conv: unsupported dtype %d / %d", x_dtype, out_dtype);
   SW_CHECK_ARG(channels > 0 && num_taps >= 1 && num_taps <= kMaxTaps && rows < (1ll << 31),
-               "short_conv: %d taps (1..%d supported), %d channels", num_taps, kMaxTaps, channels);
+               "causal_conv: %d taps (1..%d supported), %d channels", num_taps, kMaxTaps, channels);
   const dim3 grid((unsigned)rows, (unsigned)((channels + kRowThreads - 1) / kRowThreads));
-  SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(short_conv_kernel<T>, grid, dim3(kRowThreads), 0,
-                                                 static_cast<hipStream_t>(stream), out, x, x_stride, taps, state,
-                                                 q_start, ctx_len, token_seq, state_slot, channels, num_taps););
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define SWM_CONV_LAUNCH(TX, TO)                                                                                       \
+  hipLaunchKernelGGL((short_conv_kernel<TX, TO>), grid, dim3(kRowThreads), 0, s, out, x, x_stride, taps, state,       \
+                     q_start, ctx_len, token_seq, state_slot, channels, num_taps, silu, residual)
+  if (x_dtype == SW_F32) {
+    if (out_dtype == SW_F32) SWM_CONV_LAUNCH(float, float); else SWM_CONV_LAUNCH(float, sw::bf16_t);
+  } else {
+    if (out_dtype == SW_F32) SWM_CONV_LAUNCH(sw::bf16_t, float); else SWM_CONV_LAUNCH(sw::bf16_t, sw::bf16_t);
+  }
+#undef SWM_CONV_LAUNCH
   SW_CHECK_LAUNCH();
   return SW_OK;
 }

@@ -12,6 +12,7 @@
 namespace swm {
 
 constexpr int kPbThreads = 256;
+constexpr int kMaxNormHeads = 1024;     // query plus key heads of a layer whose rotation kernel also norms them
 
 // residual += (a + b + c);  out = residual / sqrt(mean(residual^2) + eps) * (offset + weight)
 template <typename T>
@@ -71,10 +72,39 @@ __global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
     float* __restrict__ q_out, const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ v,
     int64_t in_stride, const int64_t* __restrict__ positions, const float* __restrict__ inv_freq, int rot_dims,
     void* __restrict__ key_cache, void* __restrict__ value_cache, const int64_t* __restrict__ slot_mapping, int heads,
-    int kv_heads, int dim, int vdim, int pair_halves) {
+    int kv_heads, int dim, int vdim, int pair_halves, const float* __restrict__ q_norm,
+    const float* __restrict__ k_norm, float norm_eps) {
   const int64_t t = blockIdx.x;
   const int64_t row = t * in_stride;
   const float pos = (float)positions[t];
+  // optional RMS norm of every query and key head over its coordinates (one weight [dim] for all heads), before
+  // the rotation: a wave per head works out the head's factor
+  __shared__ float fac[kMaxNormHeads];
+  const bool normed = q_norm != nullptr;
+  if (normed) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int all = heads + (k != nullptr ? kv_heads : 0);
+    for (int h = wave; h < all; h += kPbThreads / 64) {
+      const void* src = h < heads ? q : k;
+      const int64_t off = row + (int64_t)(h < heads ? h : h - heads) * dim;
+      float ss = 0.0f;
+      for (int i = lane; i < dim; i += 64) {
+        const float x = ld<T>(src, off + i);
+        ss += x * x;
+      }
+      ss = sw::wave_sum(ss);
+      if (lane == 0) fac[h] = 1.0f / sqrtf(ss / (float)dim + norm_eps);
+    }
+    __syncthreads();
+  }
+  auto lq = [&](int h, int i) {
+    const float x = ld<T>(q, row + (int64_t)h * dim + i);
+    return normed ? x * fac[h] * q_norm[i] : x;
+  };
+  auto lk = [&](int h, int i) {
+    const float x = ld<T>(k, row + (int64_t)h * dim + i);
+    return normed ? x * fac[heads + h] * k_norm[i] : x;
+  };
   if (pair_halves) {
     // coordinate i < rot_dims / 2 turns with coordinate i + rot_dims / 2; those from rot_dims on pass
     const int hf = rot_dims / 2, units = dim - hf;            // a unit: one pair, or one passed-through coordinate
@@ -82,13 +112,13 @@ __global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
       const int h = e / units, u = e % units;
       const int64_t src = row + h * dim, dst = t * (int64_t)heads * dim + h * dim;
       if (u < hf) {
-        const float a = ld<T>(q, src + u), b = ld<T>(q, src + u + hf);
+        const float a = lq(h, u), b = lq(h, u + hf);
         float s, c;
         sincosf(pos * inv_freq[u], &s, &c);
         q_out[dst + u] = a * c - b * s;
         q_out[dst + u + hf] = b * c + a * s;
       } else {
-        q_out[dst + u + hf] = ld<T>(q, src + u + hf);
+        q_out[dst + u + hf] = lq(h, u + hf);
       }
     }
     if (k == nullptr) return;
@@ -98,13 +128,13 @@ __global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
       const int h = e / units, u = e % units;
       const int64_t src = row + h * dim, dst = slot * (int64_t)kv_heads * dim + h * dim;
       if (u < hf) {
-        const float a = ld<T>(k, src + u), b = ld<T>(k, src + u + hf);
+        const float a = lk(h, u), b = lk(h, u + hf);
         float s, c;
         sincosf(pos * inv_freq[u], &s, &c);
         st<T>(key_cache, dst + u, a * c - b * s);
         st<T>(key_cache, dst + u + hf, b * c + a * s);
       } else {
-        st<T>(key_cache, dst + u + hf, ld<T>(k, src + u + hf));
+        st<T>(key_cache, dst + u + hf, lk(h, u + hf));
       }
     }
     for (int e = threadIdx.x; e < kv_heads * vdim; e += kPbThreads)
@@ -116,7 +146,7 @@ __global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
   for (int e = threadIdx.x; e < heads * pairs; e += kPbThreads) {
     const int h = e / pairs, i = e % pairs;
     const int64_t src = row + h * dim + 2 * i, dst = t * (int64_t)heads * dim + h * dim + 2 * i;
-    const float a = ld<T>(q, src), b = ld<T>(q, src + 1);
+    const float a = lq(h, 2 * i), b = lq(h, 2 * i + 1);
     if (i < half) {
       float s, c;
       sincosf(pos * inv_freq[i], &s, &c);
@@ -129,14 +159,14 @@ __global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
   }
   if (dim & 1)
     for (int h = threadIdx.x; h < heads; h += kPbThreads)
-      q_out[t * (int64_t)heads * dim + h * dim + dim - 1] = ld<T>(q, row + h * dim + dim - 1);
+      q_out[t * (int64_t)heads * dim + h * dim + dim - 1] = lq(h, dim - 1);
   if (k == nullptr) return;
   const int64_t slot = slot_mapping[t];
   if (slot < 0) return;
   for (int e = threadIdx.x; e < kv_heads * pairs; e += kPbThreads) {
     const int h = e / pairs, i = e % pairs;
     const int64_t src = row + h * dim + 2 * i, dst = slot * (int64_t)kv_heads * dim + h * dim + 2 * i;
-    const float a = ld<T>(k, src), b = ld<T>(k, src + 1);
+    const float a = lk(h, 2 * i), b = lk(h, 2 * i + 1);
     if (i < half) {
       float s, c;
       sincosf(pos * inv_freq[i], &s, &c);
@@ -149,7 +179,7 @@ __global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
   }
   if (dim & 1)
     for (int h = threadIdx.x; h < kv_heads; h += kPbThreads)
-      st<T>(key_cache, slot * (int64_t)kv_heads * dim + h * dim + dim - 1, ld<T>(k, row + h * dim + dim - 1));
+      st<T>(key_cache, slot * (int64_t)kv_heads * dim + h * dim + dim - 1, lk(h, dim - 1));
   for (int e = threadIdx.x; e < kv_heads * vdim; e += kPbThreads)
     st<T>(value_cache, slot * (int64_t)kv_heads * vdim + e, ld<T>(v, row + e));
 }
@@ -159,7 +189,8 @@ constexpr int kMaxRouterExperts = 256;
 
 __global__ __launch_bounds__(256) void group_router_kernel(
     int32_t* __restrict__ chosen, float* __restrict__ weights, const float* __restrict__ logits,
-    const float* __restrict__ correction, int64_t rows, int experts, int top, int groups, int keep, float scale) {
+    const float* __restrict__ correction, int64_t rows, int experts, int top, int groups, int keep, float scale,
+    int softmax, int group_best_one, int normalize) {
   __shared__ float s_score[4][kMaxRouterExperts];
   __shared__ float s_choice[4][kMaxRouterExperts];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -167,12 +198,24 @@ __global__ __launch_bounds__(256) void group_router_kernel(
   const bool live = t < rows;
   float* score = s_score[wave];
   float* choice = s_choice[wave];
-  if (live)
+  if (live) {
+    float top_logit = 0.0f, inv_sum = 1.0f;
+    if (softmax) {                                           // scores: the softmax over ALL experts
+      float m = -INFINITY;
+      for (int e = lane; e < experts; e += 64) m = fmaxf(m, logits[t * experts + e]);
+      for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+      float sum = 0.0f;
+      for (int e = lane; e < experts; e += 64) sum += expf(logits[t * experts + e] - m);
+      top_logit = m;
+      inv_sum = 1.0f / sw::wave_sum(sum);
+    }
     for (int e = lane; e < experts; e += 64) {
-      const float s = sigmoidf_(logits[t * experts + e]);
+      const float z = logits[t * experts + e];
+      const float s = softmax ? expf(z - top_logit) * inv_sum : sigmoidf_(z);
       score[e] = s;
       choice[e] = s + (correction != nullptr ? correction[e] : 0.0f);
     }
+  }
   __syncthreads();
   if (!live) return;
   if (lane != 0) return;
@@ -192,7 +235,7 @@ __global__ __launch_bounds__(256) void group_router_kernel(
           if (c > first) { second = first; first = c; }
           else if (c > second) second = c;
         }
-        const float gs = size > 1 ? first + second : first;
+        const float gs = (size > 1 && !group_best_one) ? first + second : first;
         if (worst < 0 || gs < worst_score) { worst = g; worst_score = gs; }
       }
       dropped[worst >> 6] |= 1ull << (worst & 63);
@@ -210,7 +253,7 @@ __global__ __launch_bounds__(256) void group_router_kernel(
     weights[t * top + n] = score[best];
     total += score[best];
   }
-  const float f = scale / (total + 1e-20f);
+  const float f = normalize ? scale / (total + 1e-20f) : scale;
   for (int n = 0; n < top; ++n) weights[t * top + n] *= f;
 }
 
@@ -292,7 +335,19 @@ int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, in
                    const int64_t* positions, const float* inv_freq, int rot_dims, int pair_halves, void* key_cache,
                    void* value_cache, const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim,
                    int vdim, int act_dtype, void* stream) {
+  return swm_norm_rope_cache(q_out, q, k, v, in_stride, nullptr, nullptr, 0.0f, positions, inv_freq, rot_dims,
+                             pair_halves, key_cache, value_cache, slot_mapping, rows, heads, kv_heads, dim, vdim,
+                             act_dtype, stream);
+}
+
+int swm_norm_rope_cache(float* q_out, const void* q, const void* k, const void* v, int64_t in_stride,
+                        const float* q_norm, const float* k_norm, float norm_eps, const int64_t* positions,
+                        const float* inv_freq, int rot_dims, int pair_halves, void* key_cache, void* value_cache,
+                        const int64_t* slot_mapping, int64_t rows, int heads, int kv_heads, int dim, int vdim,
+                        int act_dtype, void* stream) {
   using namespace swm;
+  SW_CHECK_ARG(q_norm == nullptr || ((k == nullptr || k_norm != nullptr) && heads + kv_heads <= kMaxNormHeads),
+               "rope_cache: a query norm needs a key norm, and at most %d heads in all", kMaxNormHeads);
   if (rows == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(act_dtype), "rope_cache: unsupported dtype %d", act_dtype);
   SW_CHECK_ARG(heads > 0 && dim > 0 && rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0 && rows < (1ll << 31),
@@ -304,13 +359,20 @@ int swm_rope_cache(float* q_out, const void* q, const void* k, const void* v, in
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(rope_cache_kernel<T>, dim3((unsigned)rows), dim3(kPbThreads), 0,
                                                  static_cast<hipStream_t>(stream), q_out, q, k, v, in_stride, positions,
                                                  inv_freq, rot_dims, key_cache, value_cache, slot_mapping, heads,
-                                                 kv_heads, dim, vdim, pair_halves););
+                                                 kv_heads, dim, vdim, pair_halves, q_norm, k_norm, norm_eps););
   SW_CHECK_LAUNCH();
   return SW_OK;
 }
 
 int swm_group_router(int32_t* chosen, float* weights, const float* logits, const float* correction, int64_t rows,
                      int experts, int top, int groups, int keep, float scale, void* stream) {
+  return swm_group_router_as(chosen, weights, logits, correction, rows, experts, top, groups, keep, scale, 0, 0, 1,
+                             stream);
+}
+
+int swm_group_router_as(int32_t* chosen, float* weights, const float* logits, const float* correction, int64_t rows,
+                        int experts, int top, int groups, int keep, float scale, int softmax, int group_best_one,
+                        int normalize, void* stream) {
   using namespace swm;
   if (rows == 0) return SW_OK;
   SW_CHECK_ARG(experts > 0 && experts <= kMaxRouterExperts && top > 0 && top <= experts,
@@ -319,7 +381,8 @@ int swm_group_router(int32_t* chosen, float* weights, const float* logits, const
                    (int64_t)keep * (experts / groups) >= top,
                "group_router: %d groups, %d kept, %d experts, top %d", groups, keep, experts, top);
   hipLaunchKernelGGL(group_router_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     chosen, weights, logits, correction, rows, experts, top, groups, keep, scale);
+                     chosen, weights, logits, correction, rows, experts, top, groups, keep, scale, softmax, group_best_one,
+                     normalize);
   SW_CHECK_LAUNCH();
   return SW_OK;
 }

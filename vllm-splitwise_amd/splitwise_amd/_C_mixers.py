@@ -18,7 +18,7 @@ import torch
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_PKG_DIR, "libsplitwise_mixers.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 SW_F32, SW_BF16 = 0, 2
 _ACT = {torch.float32: SW_F32, torch.bfloat16: SW_BF16}
@@ -56,8 +56,15 @@ _SIGNATURES = {
     "swm_head_norm_gate_act": [_p, _p, _p, _l, _p, _i, _f, _l, _i, _i, _i, _i, _p],
     "swm_gla": [_p, _p, _p, _p, _l, _p, _l, _p, _f, _f, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
     "swm_lightning": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
+    "swm_group_norm_add": [_p, _p, _l, _f, _p, _l, _f, _i, _p, _p, _p, _p, _i, _i, _f, _l, _i, _p],
+    "swm_causal_conv": [_p, _i, _p, _i, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _p],
+    "swm_gated_delta": [_p, _p, _p, _l, _p, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
+    "swm_norm_rope_cache": [_p, _p, _p, _p, _l, _p, _p, _f, _p, _p, _i, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
+    "swm_sigmoid_attention": [_p, _p, _p, _p, _p, _l, _p, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p,
+                              _i, _p],
+    "swm_group_router_as": [_p, _p, _p, _p, _l, _i, _i, _i, _i, _f, _i, _i, _i, _p],
 }
-ACT_GELU, ACT_RELU2 = 0, 1
+ACT_GELU, ACT_RELU2, ACT_NONE = 0, 1, 2
 
 _lib = None
 
@@ -290,6 +297,56 @@ def short_conv(out: torch.Tensor, x: torch.Tensor, taps: torch.Tensor, state: to
                                           _act(x), _stream(x)))
 
 
+def causal_conv(out: torch.Tensor, x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, batch,
+                silu: bool = False, residual: bool = True) -> None:
+    """out [rows, channels] (any activation dtype) = act(conv(x) + x) (``residual``) or act(conv(x)), act = silu or
+    none; x: a 2-D view, fp32 or bf16; the state [slots, taps - 1, channels] (fp32: the sequence's last inputs) is read
+    and then moved past the step's tokens."""
+    _dev(out, x, taps, state)
+    _f32c(taps, "taps")
+    _f32c(state, "state")
+    stride = _rows(x, "x")
+    rows, channels = x.shape
+    n = _ragged_ok(batch, rows)
+    k = taps.shape[1]
+    _need(out.shape == x.shape and out.is_contiguous() and taps.shape[0] == channels
+          and state.shape[1:] == (k - 1, channels) and batch.max_state_slot < state.shape[0], "causal_conv: shapes")
+    with _on_device_of(x):
+        lib = load_library()
+        _check(lib.swm_causal_conv(out.data_ptr(), _act(out), x.data_ptr(), _act(x), stride, taps.data_ptr(),
+                                   state.data_ptr(), batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
+                                   batch.token_seq.data_ptr(), batch.state_slot.data_ptr(), rows, channels, k,
+                                   1 if silu else 0, 1 if residual else 0, _stream(x)))
+        _check(lib.swm_short_conv_advance(state.data_ptr(), x.data_ptr(), stride, batch.q_start.data_ptr(),
+                                          batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), n, channels, k,
+                                          _act(x), _stream(x)))
+
+
+def gated_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, decay_pre: torch.Tensor,
+                dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor, batch, heads: int, kv_heads: int,
+                dim: int, vdim: int) -> None:
+    """The delta rule with ONE decay per head: decay_pre, beta_pre [rows, heads] (2-D views in the activation dtype),
+    dt_bias, a_log fp32 [heads]; qkv fp32 [rows, 2 * kv_heads * dim + heads * vdim] from the short convolution;
+    state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim]."""
+    _dev(out, qkv, beta_pre, decay_pre, dt_bias, a_log, state)
+    for t, what in ((out, "out"), (qkv, "qkv"), (dt_bias, "dt_bias"), (a_log, "a_log"), (state, "state")):
+        _f32c(t, what)
+    rows = qkv.shape[0]
+    n = _ragged_ok(batch, rows)
+    _need(qkv.shape[1] == 2 * kv_heads * dim + heads * vdim and out.shape == (rows, heads * vdim)
+          and beta_pre.shape == (rows, heads) and decay_pre.shape == (rows, heads)
+          and decay_pre.dtype == beta_pre.dtype and dt_bias.numel() == heads and a_log.numel() == heads
+          and state.shape[1:] == (heads, dim, vdim) and batch.max_state_slot < state.shape[0],
+          "gated_delta: shapes")
+    work = torch.empty(rows * heads * (3 * (-(-dim // 4) * 4) + 1), dtype=torch.float32, device=qkv.device)
+    with _on_device_of(qkv):
+        _check(load_library().swm_gated_delta(
+            out.data_ptr(), qkv.data_ptr(), beta_pre.data_ptr(), _rows(beta_pre, "beta_pre"), decay_pre.data_ptr(),
+            _rows(decay_pre, "decay_pre"), dt_bias.data_ptr(), a_log.data_ptr(), state.data_ptr(),
+            batch.q_start.data_ptr(), batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), rows, n, heads, kv_heads,
+            dim, vdim, work.data_ptr(), _act(decay_pre), _stream(qkv)))
+
+
 def channel_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, decay_pre: torch.Tensor,
                   dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor, batch, heads: int, kv_heads: int,
                   dim: int, vdim: int) -> None:
@@ -356,17 +413,23 @@ def head_norm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weigh
 
 def expert_ffn(out: torch.Tensor, x: torch.Tensor, up: torch.Tensor, down: torch.Tensor, order: torch.Tensor,
                expert_start: torch.Tensor, top: int, weight: float, activation: int = ACT_GELU,
-               pair_weight: Optional[torch.Tensor] = None) -> None:
+               pair_weight: Optional[torch.Tensor] = None, glu: Optional[tuple] = None) -> None:
     """out (fp32 [rows, width], zeroed by the caller) += weight * sum over each row's experts of
     pair_weight[row, choice] * down[e] act(up[e] x[row]); ``order`` / ``expert_start``: the (row, choice) pairs
     sorted by expert and every expert's first sorted pair; ``activation``: ACT_GELU (exact gelu) or ACT_RELU2;
-    ``pair_weight`` fp32 [rows, top] (None: all 1)."""
+    ``pair_weight`` fp32 [rows, top] (None: all 1).  ``glu`` = (alpha, limit, shift): a gated hidden layer -- ``up``
+    holds every expert's gate rows and then its up rows ([experts, 2 * ff, width]) and the hidden layer is
+    g sigmoid(alpha g) (u + shift) with g = min(gate x, limit), u = clamp(up x, -limit, limit)."""
     _dev(out, x, up, down, order, expert_start, pair_weight)
     _f32c(out, "out")
     rows, width = x.shape
     experts, ff = up.shape[0], up.shape[1]
+    if glu is not None:
+        _need(ff % 2 == 0, "expert_ffn: a gated hidden layer has gate and up rows")
+        activation = ACT_NONE
     _need(x.is_contiguous() and up.is_contiguous() and down.is_contiguous() and up.dtype == x.dtype == down.dtype
-          and up.shape == (experts, ff, width) and down.shape == (experts, width, ff) and out.shape == (rows, width)
+          and up.shape == (experts, ff, width) and out.shape == (rows, width)
+          and down.shape == (experts, width, ff // 2 if glu is not None else ff)
           and order.dtype == torch.int32 and order.numel() == rows * top and order.is_contiguous()
           and expert_start.dtype == torch.int32 and expert_start.numel() == experts + 1
           and expert_start.is_contiguous(), "expert_ffn: shapes")
@@ -380,6 +443,12 @@ def expert_ffn(out: torch.Tensor, x: torch.Tensor, up: torch.Tensor, down: torch
         _check(lib.swm_expert_up(hidden.data_ptr(), x.data_ptr(), up.data_ptr(), order.data_ptr(),
                                  expert_start.data_ptr(), experts, pairs, width, ff, top, activation, _act(x),
                                  _stream(x)))
+        if glu is not None:
+            ff //= 2
+            gated = torch.empty(pairs, ff, dtype=x.dtype, device=x.device)
+            _check(lib.swm_clamped_glu(gated.data_ptr(), hidden.data_ptr(), 2 * ff, pairs, ff, float(glu[0]),
+                                       float(glu[1]), float(glu[2]), _act(x), _stream(x)))
+            hidden = gated
         _check(lib.swm_expert_down_weighted(out.data_ptr(), hidden.data_ptr(), down.data_ptr(), order.data_ptr(),
                                             expert_start.data_ptr(), experts, pairs, width, ff, top, weight,
                                             None if pair_weight is None else pair_weight.data_ptr(), _act(x),
@@ -416,6 +485,38 @@ def stream_add_norm(residual: torch.Tensor, weight: Optional[torch.Tensor], offs
             SW_F32 if act is None else _act(act), _stream(residual)))
 
 
+def group_norm_add(residual: torch.Tensor, groups: int, eps: float, y1: Optional[torch.Tensor] = None,
+                   post_weight: Optional[torch.Tensor] = None, layer_scale: Optional[torch.Tensor] = None,
+                   y2: Optional[torch.Tensor] = None, s1: float = 1.0, s2: float = 1.0,
+                   weight: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> None:
+    """N(u; w): a row in ``groups`` equal runs, each over its own root mean square, the row times w.
+    residual (fp32, in place) += layer_scale * N(s1 * y1 + s2 * y2; post_weight) (y1, y2: 2-D views of one dtype,
+    fp32 or bf16), then out = N(residual; weight) in out's dtype (fp32 or bf16)."""
+    _dev(residual, y1, y2, post_weight, layer_scale, weight, out)
+    _f32c(residual, "residual")
+    rows, width = residual.shape
+    _need(y1 is not None or out is not None, "group_norm_add: nothing to do")
+    if y1 is not None:
+        _f32c(post_weight, "post_weight")
+        _need(y1.shape == residual.shape and post_weight.numel() == width, "group_norm_add: addend")
+        if y2 is not None:
+            _need(y2.shape == residual.shape and y2.dtype == y1.dtype, "group_norm_add: second addend")
+        if layer_scale is not None:
+            _f32c(layer_scale, "layer_scale")
+            _need(layer_scale.numel() == width, "group_norm_add: layer scale")
+    else:
+        _need(y2 is None, "group_norm_add: a second addend without a first")
+    if out is not None:
+        _f32c(weight, "weight")
+        _need(out.shape == residual.shape and out.is_contiguous() and weight.numel() == width, "group_norm_add: out")
+    with _on_device_of(residual):
+        _check(load_library().swm_group_norm_add(
+            residual.data_ptr(), _opt_ptr(y1), 0 if y1 is None else _rows(y1, "y1"), s1, _opt_ptr(y2),
+            0 if y2 is None else _rows(y2, "y2"), s2, SW_F32 if y1 is None else _act(y1), _opt_ptr(post_weight),
+            _opt_ptr(layer_scale), _opt_ptr(weight), _opt_ptr(out), SW_F32 if out is None else _act(out), groups, eps,
+            rows, width, _stream(residual)))
+
+
 def clamped_glu(out: torch.Tensor, gate_up: torch.Tensor, alpha: float, limit: float, shift: float) -> None:
     """gate_up [rows, 2 * ff] = gate | up -> out [rows, ff] = g sigmoid(alpha g) (u + shift) with g = min(gate, limit),
     u = clamp(up, -limit, limit)."""
@@ -438,11 +539,20 @@ def relu2(out: torch.Tensor, x: torch.Tensor) -> None:
 def rope_cache(q_out: torch.Tensor, q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
                positions: torch.Tensor, inv_freq: Optional[torch.Tensor], heads: int, kv_heads: int, dim: int, vdim: int,
                key_cache: Optional[torch.Tensor], value_cache: Optional[torch.Tensor],
-               slot_mapping: Optional[torch.Tensor], pair_halves: bool = False) -> None:
+               slot_mapping: Optional[torch.Tensor], pair_halves: bool = False,
+               q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
+               norm_eps: float = 0.0) -> None:
     """q, k, v: column ranges of ONE projection output.  q_out fp32 = rotated q; rotated k and v go to the caches
     [pages, page, kv_heads * size] (k None: a layer that reads another layer's keys).  ``pair_halves``: coordinate i
-    turns with coordinate i + rot / 2 instead of neighbours (2i, 2i + 1)."""
-    _dev(q_out, q, k, v, positions, inv_freq, key_cache, value_cache, slot_mapping)
+    turns with coordinate i + rot / 2 instead of neighbours (2i, 2i + 1).  ``q_norm`` / ``k_norm`` (fp32 [dim]): every
+    query / key head first gets an RMS norm over its coordinates with that weight."""
+    _dev(q_out, q, k, v, positions, inv_freq, key_cache, value_cache, slot_mapping, q_norm, k_norm)
+    if q_norm is not None:
+        _f32c(q_norm, "q_norm")
+        _need(q_norm.numel() == dim, "rope_cache: query norm weight")
+        if k is not None:
+            _f32c(k_norm, "k_norm")
+            _need(k_norm.numel() == dim, "rope_cache: key norm weight")
     _f32c(q_out, "q_out")
     stride = _rows(q, "q")
     rows = q.shape[0]
@@ -467,8 +577,9 @@ def rope_cache(q_out: torch.Tensor, q: torch.Tensor, k: Optional[torch.Tensor], 
         _need(slot_mapping.dtype == torch.int64 and slot_mapping.numel() == rows and slot_mapping.is_contiguous(),
               "rope_cache: slot_mapping must be int64 [rows]")
     with _on_device_of(q):
-        _check(load_library().swm_rope_cache(
-            q_out.data_ptr(), q.data_ptr(), _opt_ptr(k), _opt_ptr(v), stride, positions.data_ptr(),
+        _check(load_library().swm_norm_rope_cache(
+            q_out.data_ptr(), q.data_ptr(), _opt_ptr(k), _opt_ptr(v), stride, _opt_ptr(q_norm),
+            _opt_ptr(k_norm) if q_norm is not None else None, norm_eps, positions.data_ptr(),
             _opt_ptr(inv_freq) if rot else None, rot, 1 if pair_halves else 0,
             None if k is None else key_cache.data_ptr(),
             None if k is None else value_cache.data_ptr(), None if k is None else slot_mapping.data_ptr(), rows, heads,
@@ -476,8 +587,11 @@ def rope_cache(q_out: torch.Tensor, q: torch.Tensor, k: Optional[torch.Tensor], 
 
 
 def group_router(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int, keep: int,
-                 scale: float):
-    """logits fp32 [rows, experts] -> (chosen int32 [rows, top], weights fp32 [rows, top])."""
+                 scale: float, softmax: bool = False, group_best_one: bool = False, normalize: bool = True):
+    """logits fp32 [rows, experts] -> (chosen int32 [rows, top], weights fp32 [rows, top]).  Scores: sigmoid of the
+    logits, or with ``softmax`` their softmax over all experts; a group scores the sum of its two best choice scores,
+    or with ``group_best_one`` its best; the chosen experts' scores are divided by their sum unless ``normalize`` is
+    off; all times ``scale``."""
     _dev(logits, correction)
     _f32c(logits, "logits")
     rows, experts = logits.shape
@@ -487,9 +601,10 @@ def group_router(logits: torch.Tensor, correction: Optional[torch.Tensor], top: 
     chosen = torch.empty(rows, top, dtype=torch.int32, device=logits.device)
     weights = torch.empty(rows, top, dtype=torch.float32, device=logits.device)
     with _on_device_of(logits):
-        _check(load_library().swm_group_router(chosen.data_ptr(), weights.data_ptr(), logits.data_ptr(),
-                                               _opt_ptr(correction), rows, experts, top, groups, keep, scale,
-                                               _stream(logits)))
+        _check(load_library().swm_group_router_as(chosen.data_ptr(), weights.data_ptr(), logits.data_ptr(),
+                                                  _opt_ptr(correction), rows, experts, top, groups, keep, scale,
+                                                  1 if softmax else 0, 1 if group_best_one else 0,
+                                                  1 if normalize else 0, _stream(logits)))
     return chosen, weights
 
 
@@ -509,13 +624,19 @@ def group_pairs(chosen: torch.Tensor, experts: int):
 
 def capped_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor, value_cache: Optional[torch.Tensor],
                      gate: Optional[torch.Tensor], batch, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
-                     softcap: float = 0.0, window: int = 0, chunk: int = 0, sink: bool = False) -> None:
+                     softcap: float = 0.0, window: int = 0, chunk: int = 0, sink: bool = False,
+                     score_bias: Optional[torch.Tensor] = None) -> None:
     """out [rows, heads * vdim] (cache dtype); q fp32 [rows, heads * dim]; caches [pages, page, kv_heads * size];
     gate (None: no gate): a 2-D view [rows, heads * vdim] in the cache dtype.  ``window`` / ``chunk``: the mask (a
     sliding window, or chunks counted from position 0; neither: plain causal); ``sink``: one more term exp(0) in the
     softmax's denominator.  ``value_cache`` None: a token's values are the first kv_heads * vdim elements of its
-    key row (attention over a shared latent)."""
-    _dev(out, q, key_cache, value_cache, gate)
+    key row (attention over a shared latent).  ``score_bias`` (fp32 [heads]): no softmax -- a seen key weighs
+    sigmoid(score + score_bias[head]) and the weights are not normalised (window mask only)."""
+    _dev(out, q, key_cache, value_cache, gate, score_bias)
+    if score_bias is not None:
+        _f32c(score_bias, "score_bias")
+        _need(score_bias.numel() == heads and not softcap and not chunk and not sink,
+              "capped_attention: sigmoid weights take a bias per head and no cap, chunks or sink")
     _f32c(q, "q")
     rows = q.shape[0]
     n = _ragged_ok(batch, rows)
@@ -545,6 +666,15 @@ def capped_attention(out: torch.Tensor, q: torch.Tensor, key_cache: torch.Tensor
         need = lib.swm_masked_attention_workspace_floats(rows, n, longest, heads, kv_heads, vdim, key_cache.shape[1],
                                                          tables.shape[1], int(window), int(chunk))
         work = torch.empty(need, dtype=torch.float32, device=q.device) if need > 0 else None
+        if score_bias is not None:
+            _need(k_stride == kv_heads * dim and v_stride == kv_heads * vdim and value_cache is not key_cache,
+                  "capped_attention: sigmoid weights read plain key and value caches")
+            _check(lib.swm_sigmoid_attention(
+                out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), _opt_ptr(gate),
+                0 if gate is None else _rows(gate, "gate"), score_bias.data_ptr(), tables.data_ptr(), tables.shape[1],
+                batch.q_start.data_ptr(), batch.ctx_len.data_ptr(), rows, n, longest, heads, kv_heads, dim, vdim,
+                key_cache.shape[1], scale, int(window), _opt_ptr(work), _act(out), _stream(q)))
+            return
         _check(lib.swm_masked_attention(
             out.data_ptr(), q.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), _opt_ptr(gate),
             0 if gate is None else _rows(gate, "gate"), tables.data_ptr(), tables.shape[1], batch.q_start.data_ptr(),
@@ -708,4 +838,5 @@ ops = SimpleNamespace(expert_ffn=expert_ffn, ACT_GELU=ACT_GELU, ACT_RELU2=ACT_RE
     general_delta=general_delta, head_norm_gate=head_norm_gate, stream_add_norm=stream_add_norm,
     clamped_glu=clamped_glu, relu2=relu2, rope_cache=rope_cache, group_router=group_router, group_pairs=group_pairs,
     capped_attention=capped_attention, lightning=lightning, gated_stream_step=gated_stream_step, poly_norm=poly_norm,
-    gate_mul=gate_mul, latent_rope_cache=latent_rope_cache, gla=gla)
+    gate_mul=gate_mul, latent_rope_cache=latent_rope_cache, gla=gla, ACT_NONE=ACT_NONE,
+    group_norm_add=group_norm_add, causal_conv=causal_conv, gated_delta=gated_delta)

@@ -199,6 +199,9 @@ class ModelConfig:
             if raw.get("architecture") == "Lalasun":
                 from .model_executor.models.lalasun import normalize_config
                 return normalize_config(raw)
+            if raw.get("architecture") == "Bogetar":
+                from .model_executor.models.bogetar import normalize_config
+                return normalize_config(raw)
             arch = (raw.get("architectures") or [""])[0].lower()
             raw["architecture"] = "opt" if "opt" in arch else "llama"
             raw.setdefault("num_key_value_heads", raw["num_attention_heads"])

@@ -307,6 +307,53 @@ class CappedGatedAttention(nn.Module):
         return out
 
 
+class SigmoidWindowAttention(nn.Module):
+    """Attention WITHOUT a softmax, grouped query heads over a paged cache: a key that a position sees weighs
+    sigmoid((q . k) * scale + bias[head]) with one learned bias per query head, and the weights are not normalised
+    over the keys.  Queries and keys get an RMS norm per head over their coordinates (one weight [dim] shared by the
+    heads, ``qk_norm_eps`` None: no norm), then a partial rotary embedding on the pairs (i, i + rot / 2) (or
+    neighbours); position i sees j with 0 <= i - j < ``window`` (0: every j <= i); optionally a sigmoid gate on the
+    concatenated heads.  Keys are cached after norm and rotation; caches are [pages, page, kv_heads * size].  Scores,
+    weights and sums are fp32."""
+
+    def __init__(self, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 inv_freq: Optional[torch.Tensor] = None, window: int = 0, qk_norm_eps: Optional[float] = None,
+                 pair_halves: bool = True) -> None:
+        super().__init__()
+        assert heads % kv_heads == 0
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.window, self.pair_halves, self.qk_norm_eps = float(scale), int(window), pair_halves, qk_norm_eps
+        freqs = torch.zeros(0, dtype=torch.float32) if inv_freq is None else inv_freq.to(torch.float32)
+        assert 2 * freqs.numel() <= dim
+        self.register_buffer("inv_freq", freqs.clone(), persistent=False)     # a constant of the config, not a weight
+        self.score_bias = nn.Parameter(torch.zeros(heads, dtype=torch.float32), requires_grad=False)
+        self.q_norm = self.k_norm = None
+        if qk_norm_eps is not None:
+            self.q_norm = nn.Parameter(torch.ones(dim, dtype=torch.float32), requires_grad=False)
+            self.k_norm = nn.Parameter(torch.ones(dim, dtype=torch.float32), requires_grad=False)
+
+    def cache_shapes(self, block_size: int):
+        """Per page: keys, values."""
+        return [(block_size, self.kv_heads * self.dim), (block_size, self.kv_heads * self.vdim)]
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: Optional[torch.Tensor],
+                positions: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                md: InputMetadata) -> torch.Tensor:
+        """q, k, v, gate: column ranges of one projection output [rows, *].  -> [rows, heads * vdim]."""
+        rows = q.shape[0]
+        q32 = torch.empty(rows, self.heads * self.dim, dtype=torch.float32, device=q.device)
+        normed = self.q_norm is not None
+        _C.mixer_ops.rope_cache(q32, q, k, v, positions, self.inv_freq, self.heads, self.kv_heads, self.dim, self.vdim,
+                                key_cache, value_cache, md.slot_mapping, self.pair_halves,
+                                self.q_norm.data if normed else None, self.k_norm.data if normed else None,
+                                self.qk_norm_eps if normed else 0.0)
+        out = torch.empty(rows, self.heads * self.vdim, dtype=q.dtype, device=q.device)
+        _C.mixer_ops.capped_attention(out, q32, key_cache, value_cache, gate, md.ragged, self.heads, self.kv_heads,
+                                      self.dim, self.vdim, self.scale, 0.0, self.window,
+                                      score_bias=self.score_bias.data)
+        return out
+
+
 class LatentAttention(nn.Module):
     """Softmax attention whose keys and values of ALL heads are linear maps of one small latent per token, plus one
     rotated key part shared by the heads:

@@ -154,6 +154,63 @@ class OffsetRMSNorm(nn.Module):
         return self.add_norm(x, out_dtype)
 
 
+class GroupRMSNorm(nn.Module):
+    """RMS norm in groups of channels: the row is cut into ``groups`` equal runs, every run is divided by its own
+    sqrt(mean(run^2) + eps), and the row is multiplied by a per-channel weight (kept in fp32).  Reads an fp32 stream.
+    For layers that norm a sublayer's input AND its output, ``add_norm`` takes the sublayer's output through this
+    norm (as the norm AFTER the sublayer) into the stream, times an optional per-channel layer scale, and writes the
+    norm of the new stream that the next sublayer reads -- one launch."""
+
+    def __init__(self, width: int, groups: int = 1, eps: float = 1e-6) -> None:
+        super().__init__()
+        if width % groups != 0:
+            raise ValueError(f"a norm over {width} channels cannot be cut into {groups} equal groups")
+        self.weight = nn.Parameter(torch.ones(width, dtype=torch.float32), requires_grad=False)
+        self.groups, self.variance_epsilon = int(groups), eps
+
+    def _forward(self, x: torch.Tensor) -> torch.Tensor:
+        parts = x.float().unflatten(-1, (self.groups, -1))
+        parts = parts * torch.rsqrt(parts.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return parts.flatten(-2) * self.weight
+
+    def forward(self, stream: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        out = torch.empty(stream.shape, dtype=out_dtype, device=stream.device)
+        _C.mixer_ops.group_norm_add(stream, self.groups, self.variance_epsilon, weight=self.weight.data, out=out)
+        return out
+
+    def add_norm(self, stream: torch.Tensor, y: torch.Tensor, layer_scale: Optional[torch.Tensor],
+                 next_norm: Optional["GroupRMSNorm"], out_dtype: torch.dtype, y2: Optional[torch.Tensor] = None,
+                 s1: float = 1.0, s2: float = 1.0) -> Optional[torch.Tensor]:
+        """stream (fp32, in place) += layer_scale * self(s1 * y + s2 * y2);  -> next_norm(stream) in ``out_dtype``
+        (None without a next norm)."""
+        out = None
+        if next_norm is not None:
+            assert next_norm.groups == self.groups and next_norm.variance_epsilon == self.variance_epsilon
+            out = torch.empty(stream.shape, dtype=out_dtype, device=stream.device)
+        _C.mixer_ops.group_norm_add(stream, self.groups, self.variance_epsilon, y, self.weight.data, layer_scale, y2,
+                                    s1, s2, None if next_norm is None else next_norm.weight.data, out)
+        return out
+
+
+class CausalConvResidual(nn.Module):
+    """A sublayer's input plus its own short causal convolution over time, per channel, no bias, no activation:
+    out_t = x_t + sum_j taps[:, j] x_(t - T + 1 + j), rows before the sequence's start counting as zeros.  The last
+    T - 1 inputs of every sequence are part of its state (``state_shape`` per slot, fp32)."""
+
+    def __init__(self, channels: int, taps: int) -> None:
+        super().__init__()
+        self.channels, self.num_taps = channels, int(taps)
+        self.taps = nn.Parameter(torch.zeros(channels, taps, dtype=torch.float32), requires_grad=False)
+
+    def state_shape(self) -> Tuple[int, int]:
+        return (self.num_taps - 1, self.channels)
+
+    def forward(self, x: torch.Tensor, state: torch.Tensor, md, out_dtype: torch.dtype) -> torch.Tensor:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _C.mixer_ops.causal_conv(out, x, self.taps.data, state, md.ragged, silu=False, residual=True)
+        return out
+
+
 class DynamicTanhNorm(nn.Module):
     """Element-wise norm without statistics of the row: out = tanh(alpha * x) * w + b, one number alpha, per-channel
     w and b, all kept in fp32; reads an fp32 stream and writes activations.  ``gated_add_norm`` first takes a

@@ -7,7 +7,11 @@ shared expert of the same form runs for every token and is added after a per-tok
 ``GroupRoutedExperts``: a learned sigmoid router in fp32 with a selection bias that enters the choice but not the
 weights, a choice limited to the best groups of neighbouring experts, weights normalised over the chosen experts
 and scaled; an expert is down(relu(up x)^2); an optional shared expert of the same form is returned beside the
-routed sum so that the caller's residual add can take both.
+routed sum so that the caller's residual add can take both.  The same layer, by its options, is a SOFTMAX router
+(``score="softmax"``: scores are the softmax over all experts), whose groups score their best expert
+(``group_score="max"``), whose weights are the chosen scores as they are (``normalize=False``) and whose experts have
+a gated hidden layer with limits (``activation="clamped_glu"``: g = min(gate x, limit), u = clamp(up x, +-limit),
+g sigmoid(alpha g) (u + 1)).
 
 Rows are grouped by expert on the device (a stable sort of the (row, choice) pairs by expert id, then a binary
 search for every expert's first pair), so each expert's rows are one contiguous run and the host never waits.
@@ -76,8 +80,17 @@ def group_pairs_by_expert(experts: torch.Tensor, num_experts: int):
 
 class GroupRoutedExperts(nn.Module):
     def __init__(self, width: int, num_experts: int, top: int, ff: int, shared_ff: Optional[int], groups: int,
-                 keep_groups: int, scale: float, dtype: torch.dtype, linear_method=None) -> None:
+                 keep_groups: int, scale: float, dtype: torch.dtype, linear_method=None, score: str = "sigmoid",
+                 group_score: str = "top2", normalize: bool = True, activation: str = "relu2",
+                 limit: float = float("inf"), glu_alpha: float = 1.702) -> None:
         super().__init__()
+        if score not in ("sigmoid", "softmax") or group_score not in ("top2", "max") or \
+                activation not in ("relu2", "clamped_glu"):
+            raise ValueError(f"unknown router score {score!r}, group score {group_score!r} or activation {activation!r}")
+        if activation == "clamped_glu" and shared_ff:
+            raise NotImplementedError("a shared expert with a gated hidden layer")
+        self.softmax, self.group_best_one, self.normalize = score == "softmax", group_score == "max", bool(normalize)
+        self.glu = (float(glu_alpha), float(limit), 1.0) if activation == "clamped_glu" else None
         if num_experts % groups != 0 or not (1 <= keep_groups <= groups) or keep_groups * (num_experts // groups) < top:
             raise ValueError(f"{num_experts} experts in {groups} groups with {keep_groups} kept cannot give {top} choices")
         self.width, self.num_experts, self.top, self.ff = width, num_experts, top, ff
@@ -85,7 +98,9 @@ class GroupRoutedExperts(nn.Module):
         # the router is fp32 whatever the model's dtype
         self.router = nn.Parameter(torch.zeros(num_experts, width, dtype=torch.float32), requires_grad=False)
         self.correction = nn.Parameter(torch.zeros(num_experts, dtype=torch.float32), requires_grad=False)
-        self.up = nn.Parameter(torch.empty(num_experts, ff, width, dtype=dtype), requires_grad=False)
+        # a gated hidden layer: every expert's gate rows, then its up rows
+        self.up = nn.Parameter(torch.empty(num_experts, (2 if self.glu else 1) * ff, width, dtype=dtype),
+                               requires_grad=False)
         self.down = nn.Parameter(torch.empty(num_experts, width, ff, dtype=dtype), requires_grad=False)
         self.shared_ff = shared_ff
         if shared_ff:
@@ -97,11 +112,12 @@ class GroupRoutedExperts(nn.Module):
         # fp32 products with the fp32 router (the library's GEMM; no reduced-precision matrix mode is switched on)
         logits = torch.matmul(h.float(), self.router.data.t())
         chosen, weights = _C.mixer_ops.group_router(logits, self.correction.data, self.top, self.groups,
-                                                    self.keep_groups, self.scale)
+                                                    self.keep_groups, self.scale, self.softmax, self.group_best_one,
+                                                    self.normalize)
         order, start = group_pairs_by_expert(chosen, self.num_experts)
         out = torch.zeros(h.shape[0], self.width, dtype=torch.float32, device=h.device)
         _C.mixer_ops.expert_ffn(out, h, self.up.data, self.down.data, order, start, self.top, 1.0,
-                                activation=_C.mixer_ops.ACT_RELU2, pair_weight=weights)
+                                activation=_C.mixer_ops.ACT_RELU2, pair_weight=weights, glu=self.glu)
         shared = None
         if self.shared_ff:
             hidden = self.shared_up(h)
@@ -114,7 +130,11 @@ class GroupRoutedExperts(nn.Module):
         self.router.data.copy_(w["router"].float())
         if "correction" in w:
             self.correction.data.copy_(w["correction"].float())
-        self.up.data.copy_(torch.stack([w[f"e{e}.up"] for e in range(self.num_experts)]))
+        if self.glu:
+            self.up.data.copy_(torch.stack([torch.cat([w[f"e{e}.gate"], w[f"e{e}.up"]], 0)
+                                            for e in range(self.num_experts)]))
+        else:
+            self.up.data.copy_(torch.stack([w[f"e{e}.up"] for e in range(self.num_experts)]))
         self.down.data.copy_(torch.stack([w[f"e{e}.down"] for e in range(self.num_experts)]))
         if self.shared_ff:
             self.shared_up.weight.data.copy_(w["shared.up"])

@@ -9,6 +9,8 @@ projections (decays, step sizes, gates, unit norms, the state itself) is fp32 in
 Delta rule, per head, S [key size, value size] (keys index rows):
   ``ChannelDeltaMixer``   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
                           g = exp(-exp(A_log) softplus(low-rank(h) + dt_bias)) per head and key channel
+  ``GatedDeltaMixer``     the same rule with ONE decay per head: g = exp(-exp(A_log) softplus(W_a h + dt_bias));
+                          the gate on the normed output is silu(W_g h)
   ``GeneralDeltaMixer``   S <- diag(w) S - (a * u)(u^T S) + k v^T;  o = S^T r,  u = k / |k|
                           w = exp(-e^(-1/2) sigmoid(low-rank-tanh(h) + w0)),  a = sigmoid(W_a h + b)
 
@@ -82,6 +84,56 @@ class ChannelDeltaMixer(nn.Module):
         self.gate_up.weight.data.copy_(w["g2"])
         self.o_proj.weight.data.copy_(w["o"])
         self.conv_taps.data.copy_(torch.cat([w["q.conv"], w["k.conv"], w["v.conv"]], 0).float().to(dev))
+        self.dt_bias.data.copy_(w["dt_bias"].float())
+        self.a_log.data.copy_(w["A_log"].float())
+        self.out_norm.data.copy_(w["norm"].float())
+
+
+class GatedDeltaMixer(nn.Module):
+    """Delta rule with a gate beta and one decay per head (see the module's docstring).  q | k | v | beta | decay |
+    output gate are one GEMM of the layer's input; q, k, v pass a short causal convolution per channel and silu; q and
+    k are made unit vectors per head inside the kernel (q also times dim^-1/2); value head h reads q / k head
+    h // (heads / kv_heads).  Each head's output gets an RMS norm over its value channels with ONE weight [vdim]
+    shared by the heads, times silu(gate), then the output projection."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, conv_taps: int, eps: float,
+                 dtype: torch.dtype, linear_method=None) -> None:
+        super().__init__()
+        assert heads % kv_heads == 0
+        self.heads, self.kv_heads, self.dim, self.vdim, self.taps, self.eps = heads, kv_heads, dim, vdim, conv_taps, eps
+        self.conv_channels = 2 * kv_heads * dim + heads * vdim          # q | k | v
+        self.in_sizes = [kv_heads * dim, kv_heads * dim, heads * vdim, heads, heads, heads * vdim]
+        self.in_proj = MergedColumnParallelLinear(width, self.in_sizes, False, dtype, linear_method)
+        self.o_proj = RowParallelLinear(heads * vdim, width, False, dtype, linear_method)
+        self.conv_taps = _f32_param(self.conv_channels, conv_taps)
+        self.dt_bias = _f32_param(heads)
+        self.a_log = _f32_param(heads)
+        self.out_norm = nn.Parameter(torch.ones(vdim, dtype=torch.float32), requires_grad=False)
+
+    def state_shapes(self) -> List[Tuple[int, ...]]:
+        """Per slot: the convolution's last inputs, the delta-rule state."""
+        return [(self.taps - 1, self.conv_channels), (self.heads, self.dim, self.vdim)]
+
+    def forward(self, h: torch.Tensor, state: List[torch.Tensor], md: InputMetadata) -> torch.Tensor:
+        conv_state, rule_state = state
+        batch = md.ragged
+        rows, c, H = h.shape[0], self.conv_channels, self.heads
+        proj = self.in_proj(h)
+        qkv = torch.empty(rows, c, dtype=torch.float32, device=h.device)
+        _C.mixer_ops.short_conv(qkv, proj[:, :c], self.conv_taps.data, conv_state, batch)
+        o = torch.empty(rows, H * self.vdim, dtype=torch.float32, device=h.device)
+        _C.mixer_ops.gated_delta(o, qkv, proj[:, c:c + H], proj[:, c + H:c + 2 * H], self.dt_bias.data, self.a_log.data,
+                                 rule_state, batch, H, self.kv_heads, self.dim, self.vdim)
+        gated = torch.empty(rows, H * self.vdim, dtype=h.dtype, device=h.device)
+        _C.mixer_ops.head_norm_gate(gated, o, proj[:, c + 2 * H:], self.out_norm.data, False, self.eps, H, self.vdim,
+                                    gate_silu=True)
+        return self.o_proj(gated)
+
+    def load_named(self, w: Dict[str, torch.Tensor]) -> None:
+        """``w``: q, q.conv, k, k.conv, v, v.conv, b, a, dt_bias, A_log, g, norm, o."""
+        self.in_proj.weight.data.copy_(torch.cat([w["q"], w["k"], w["v"], w["b"], w["a"], w["g"]], 0))
+        self.o_proj.weight.data.copy_(w["o"])
+        self.conv_taps.data.copy_(torch.cat([w["q.conv"], w["k.conv"], w["v.conv"]], 0).float())
         self.dt_bias.data.copy_(w["dt_bias"].float())
         self.a_log.data.copy_(w["A_log"].float())
         self.out_norm.data.copy_(w["norm"].float())
@@ -172,17 +224,21 @@ class GatedLinearAttentionMixer(nn.Module):
     low-rank projection of the layer's input plus a bias.  q | k | v | gate | first decay factor (| ``extra_out``
     more columns for the caller, e.g. a gate on the layer's output) are one GEMM; the decay's logarithm, the
     recurrence and the output norm are fp32.  Each head's output gets an RMS norm over its value channels with ONE
-    weight [vdim] shared by the heads, times silu(gate), then the output projection."""
+    weight [vdim] shared by the heads, times silu(gate), then the output projection.  Built with ``project=False``
+    the mixer owns neither the input nor the output projection: a layer that runs it beside another mixer on ONE
+    input GEMM hands the column ranges to ``core`` and projects the result itself."""
 
     def __init__(self, width: int, heads: int, dim: int, vdim: int, decay_rank: int, tau: float, eps: float,
-                 dtype: torch.dtype, linear_method=None, extra_out: int = 0) -> None:
+                 dtype: torch.dtype, linear_method=None, extra_out: int = 0, project: bool = True) -> None:
         super().__init__()
         self.heads, self.dim, self.vdim, self.tau, self.eps = heads, dim, vdim, float(tau), eps
         self.in_sizes = [heads * dim, heads * dim, heads * vdim, heads * vdim, decay_rank] + \
             ([extra_out] if extra_out else [])
-        self.in_proj = MergedColumnParallelLinear(width, self.in_sizes, bool(extra_out), dtype, linear_method)
+        self.in_proj = self.o_proj = None
+        if project:
+            self.in_proj = MergedColumnParallelLinear(width, self.in_sizes, bool(extra_out), dtype, linear_method)
+            self.o_proj = RowParallelLinear(heads * vdim, width, False, dtype, linear_method)
         self.decay_up = ColumnParallelLinear(decay_rank, heads * dim, False, dtype, linear_method)
-        self.o_proj = RowParallelLinear(heads * vdim, width, False, dtype, linear_method)
         self.decay_bias = _f32_param(heads * dim)
         self.out_norm = nn.Parameter(torch.ones(vdim, dtype=torch.float32), requires_grad=False)
 
@@ -191,29 +247,38 @@ class GatedLinearAttentionMixer(nn.Module):
 
     def forward(self, h: torch.Tensor, state: List[torch.Tensor], md: InputMetadata):
         """-> (output [rows, width], the ``extra_out`` columns of the input projection or None)."""
-        rows = h.shape[0]
         proj = self.in_proj(h)
         nk, nv, rank = self.heads * self.dim, self.heads * self.vdim, self.in_sizes[4]
         lo = 2 * nk + 2 * nv
-        decay_pre = self.decay_up(proj[:, lo:lo + rank])
-        o = torch.empty(rows, nv, dtype=torch.float32, device=h.device)
-        _C.mixer_ops.gla(o, proj[:, :nk], proj[:, nk:2 * nk], proj[:, 2 * nk:2 * nk + nv], decay_pre,
-                         self.decay_bias.data, self.tau, self.dim ** -0.5, state[0], md.ragged, self.heads, self.dim,
-                         self.vdim)
-        gated = torch.empty(rows, nv, dtype=h.dtype, device=h.device)
-        _C.mixer_ops.head_norm_gate(gated, o, proj[:, 2 * nk + nv:lo], self.out_norm.data, False, self.eps, self.heads,
-                                    self.vdim, gate_silu=True)
+        gated = self.core(proj[:, :nk], proj[:, nk:2 * nk], proj[:, 2 * nk:2 * nk + nv], proj[:, 2 * nk + nv:lo],
+                          proj[:, lo:lo + rank], state[0], md)
         extra = proj[:, lo + rank:] if len(self.in_sizes) > 5 else None
         return self.o_proj(gated), extra
 
+    def core(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor, decay_low: torch.Tensor,
+             state: torch.Tensor, md: InputMetadata) -> torch.Tensor:
+        """q, k, v, gate, decay_low (the decay's first, low-rank factor): column ranges of ONE projection output.
+        -> the normed, gated heads [rows, heads * vdim] in the activation dtype, before the output projection."""
+        rows, nv = q.shape[0], self.heads * self.vdim
+        decay_pre = self.decay_up(decay_low)
+        o = torch.empty(rows, nv, dtype=torch.float32, device=q.device)
+        _C.mixer_ops.gla(o, q, k, v, decay_pre, self.decay_bias.data, self.tau, self.dim ** -0.5, state, md.ragged,
+                         self.heads, self.dim, self.vdim)
+        gated = torch.empty(rows, nv, dtype=q.dtype, device=q.device)
+        _C.mixer_ops.head_norm_gate(gated, o, gate, self.out_norm.data, False, self.eps, self.heads, self.vdim,
+                                    gate_silu=True)
+        return gated
+
     def load_named(self, w: Dict[str, torch.Tensor], extra: Dict[str, torch.Tensor] = None) -> None:
-        """``w``: q, k, v, g, a1, a2, a2.b, norm, o; ``extra``: weight / bias of the ``extra_out`` columns."""
-        parts = [w["q"], w["k"], w["v"], w["g"], w["a1"]] + ([extra["weight"]] if extra else [])
-        self.in_proj.weight.data.copy_(torch.cat(parts, 0))
-        if extra:
-            self.in_proj.bias.data.zero_()
-            self.in_proj.bias.data[-extra["bias"].numel():].copy_(extra["bias"])
+        """``w``: q, k, v, g, a1, a2, a2.b, norm, o; ``extra``: weight / bias of the ``extra_out`` columns.  A mixer
+        without projections of its own takes a2, a2.b and norm."""
+        if self.in_proj is not None:
+            parts = [w["q"], w["k"], w["v"], w["g"], w["a1"]] + ([extra["weight"]] if extra else [])
+            self.in_proj.weight.data.copy_(torch.cat(parts, 0))
+            if extra:
+                self.in_proj.bias.data.zero_()
+                self.in_proj.bias.data[-extra["bias"].numel():].copy_(extra["bias"])
+            self.o_proj.weight.data.copy_(w["o"])
         self.decay_up.weight.data.copy_(w["a2"])
         self.decay_bias.data.copy_(w["a2.b"].float())
-        self.o_proj.weight.data.copy_(w["o"])
         self.out_norm.data.copy_(w["norm"].float())

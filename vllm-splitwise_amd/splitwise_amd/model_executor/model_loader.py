@@ -13,6 +13,7 @@ import torch
 import torch.nn as nn
 
 from ..config import ModelConfig
+from .models.bogetar import BogetarForCausalLM
 from .models.lalasun import LalasunForCausalLM
 from .models.lapilorn import LapilornForCausalLM
 from .models.llama import LlamaForCausalLM
@@ -20,7 +21,7 @@ from .models.nepevik import NepevikForCausalLM
 from .models.opt import OPTForCausalLM
 
 _ARCH = {"llama": LlamaForCausalLM, "opt": OPTForCausalLM, "nepevik": NepevikForCausalLM,
-         "lapilorn": LapilornForCausalLM, "lalasun": LalasunForCausalLM}
+         "lapilorn": LapilornForCausalLM, "lalasun": LalasunForCausalLM, "bogetar": BogetarForCausalLM}
 
 
 def architecture_class(name: str):

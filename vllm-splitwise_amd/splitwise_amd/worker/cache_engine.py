@@ -123,8 +123,8 @@ class CacheEngine:
 
 
 class LayeredCacheEngine:
-    """Caches of a model whose layers differ (``ModelConfig.get_cache_layout``): per layer either pages of its
-    own shapes (the model's dtype), per-sequence state slots (fp32), or the tensors of an earlier layer.
+    """Caches of a model whose layers differ (``ModelConfig.get_cache_layout``): per layer pages of its
+    own shapes (the model's dtype), per-sequence state slots (fp32), both, or the tensors of an earlier layer.
 
     ``gpu_cache[i]`` is the list of tensors that layer i's mixer receives: paged tensors are
     [num_blocks, *shape per page], state tensors [num_slots, *shape per slot].  Pages are handed out by the
@@ -154,11 +154,12 @@ class LayeredCacheEngine:
         for spec in layout:
             if "alias" in spec:
                 cache.append(cache[spec["alias"]])
-            elif "paged" in spec:
-                cache.append([torch.zeros((num_blocks, *shape), dtype=dtype, device=device) for shape in spec["paged"]])
             else:
-                cache.append([torch.zeros((num_slots, *shape), dtype=torch.float32, device=device)
-                              for shape in spec["state"]])
+                # a layer may hold both: its paged tensors come first, then its state tensors
+                cache.append([torch.zeros((num_blocks, *shape), dtype=dtype, device=device)
+                              for shape in spec.get("paged", ())] +
+                             [torch.zeros((num_slots, *shape), dtype=torch.float32, device=device)
+                              for shape in spec.get("state", ())])
         return cache
 
     def swap_in(self, src_to_dst) -> None:
