@@ -124,6 +124,34 @@ _LALASUN_PRESETS = {
     "lalasun-2k": (2048, 2, 16, 4, 4224),          # up + down of 4224 = gate + up + down of 2816
     "lalasun-4k": (4096, 2, 32, 8, 8448),
 }
+def _bogetar_preset(width: int, repeats: int, heads: int, kv_heads: int, experts: int, top: int, ff: int) -> dict:
+    """A Bogetar stack of layer sizes that resemble a served model's: per repeat three parallel layers (attention with
+    sigmoid weights over a window of 1024 beside gated linear attention) and two delta layers, each with routed experts
+    but the last, which has no feed-forward."""
+    d = width // heads
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024},
+            "rot": {"base": 10000.0, "dims": d // 2}}
+    right = {"heads": heads // 4, "dim": d // 2, "vdim": d, "tau": 16.0, "decay_rank": 32}
+    par = {"left": left, "right": right, "left_scale": 0.8, "right_scale": 0.5}
+    delta = {"heads": heads, "kv_heads": heads // 2, "dim": d, "vdim": d, "conv": 4}
+    moe = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0},
+           "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}}
+    layers = []
+    for _ in range(repeats):
+        layers += [{"type": "parallel", "mixer": par, "mlp": moe}, {"type": "delta", "mixer": delta, "mlp": moe},
+                   {"type": "parallel", "mixer": par, "mlp": moe}, {"type": "parallel", "mixer": par, "mlp": moe},
+                   {"type": "delta", "mixer": delta, "mlp": None}]
+    import copy
+    from .model_executor.models.bogetar import normalize_config
+    return normalize_config({"architecture": "Bogetar", "canon": {"taps": 4}, "layers": copy.deepcopy(layers),
+                             "norm": {"eps": 1e-6, "groups": 8}, "vocab": 32000, "width": width})
+
+
+_BOGETAR_PRESETS = {
+    # name: (width, repeats of the 5-layer pattern, heads, kv heads, experts, top, expert ff)
+    "bogetar-2k": (2048, 2, 16, 4, 32, 2, 1408),   # 2 experts of gate + up + down 1408 = the Llama stack's 2816
+    "bogetar-4k": (4096, 2, 32, 8, 32, 2, 2816),
+}
 # Llama stacks of the same width, depth and active feed-forward size, to measure the above against
 MODEL_PRESETS.update({
     "llama-2k": dict(architecture="llama", vocab_size=32000, hidden_size=2048, num_hidden_layers=10,
@@ -186,6 +214,8 @@ class ModelConfig:
             return _lapilorn_preset(*_LAPILORN_PRESETS[name])
         if name in _LALASUN_PRESETS:
             return _lalasun_preset(*_LALASUN_PRESETS[name])
+        if name in _BOGETAR_PRESETS:
+            return _bogetar_preset(*_BOGETAR_PRESETS[name])
         cfg_path = os.path.join(model, "config.json")
         if os.path.isfile(cfg_path):
             with open(cfg_path) as f:
