@@ -112,11 +112,11 @@ def parse_args():
                     help="N > 1: legs after the headline leg are skipped once the run has taken this long")
     ap.add_argument("--leg-timeout", type=float, default=600.0, help="N > 1: longest any one leg may take (s)")
     ap.add_argument("--mixers", action="store_true",
-                    help="instead of the headline workload: prefill / decode throughput of a Nepevik (or, with --mixer-family, Lapilorn) stack beside a Llama "
+                    help="instead of the headline workload: prefill / decode throughput of a Nepevik (or, with --mixer-family, Lapilorn, Lalasun, Bogetar) stack beside a Llama "
                          "stack of equal size (random weights), and the mixer kernels beside the like Llama kernels with "
                          "their distances from the roofline; one JSON line")
     ap.add_argument("--mixer-sizes", default="2k", help="with --mixers: comma-separated preset sizes (2k, 4k)")
-    ap.add_argument("--mixer-family", default="nepevik", choices=["nepevik", "lapilorn", "lalasun"],
+    ap.add_argument("--mixer-family", default="nepevik", choices=["nepevik", "lapilorn", "lalasun", "bogetar"],
                     help="with --mixers: the family of listed-layer decoders to measure beside Llama")
     ap.add_argument("--replica", default=None, help=argparse.SUPPRESS)          # set by the launcher
     ap.add_argument("--worker-cls", default=None, help=argparse.SUPPRESS)       # CPU dry runs of the launcher

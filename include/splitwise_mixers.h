@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SWM_ABI_VERSION 4
+#define SWM_ABI_VERSION 5
 int swm_abi_version(void);
 const char* swm_last_error(void);
 
@@ -139,9 +139,17 @@ int swm_expert_down(float* out, const void* hidden, const void* down, const int3
 #define SWM_ACT_GELU 0
 #define SWM_ACT_RELU2 1
 #define SWM_ACT_NONE 2 /* the products as they are: the hidden layer's gated unit is a kernel of its own */
+#define SWM_ACT_CLAMPED_GLU 3 /* swm_expert_up_as only: a gated hidden layer with limits in the kernel's epilogue */
 int swm_expert_up(void* hidden, const void* x, const void* up, const int32_t* order, const int32_t* expert_start,
                   int num_experts, int64_t sorted_rows, int width, int ff, int top, int activation, int act_dtype,
                   void* stream);
+/* swm_expert_up with the gated unit of swm_clamped_glu in its epilogue (activation SWM_ACT_CLAMPED_GLU; the other
+ * activations ignore the three numbers): `up` then holds 32 * ceil(ff / 16) rows per expert -- per run of 16 hidden
+ * channels its 16 gate rows followed by its 16 up rows, a shorter last run padded with zero rows -- and
+ * hidden[pair, c] = g sigmoid(glu_alpha g) (u + glu_shift), g = min(gate x, glu_limit), u = clamp(up x, +-glu_limit). */
+int swm_expert_up_as(void* hidden, const void* x, const void* up, const int32_t* order, const int32_t* expert_start,
+                     int num_experts, int64_t sorted_rows, int width, int ff, int top, int activation, float glu_alpha,
+                     float glu_limit, float glu_shift, int act_dtype, void* stream);
 int swm_expert_down_weighted(float* out, const void* hidden, const void* down, const int32_t* order,
                              const int32_t* expert_start, int num_experts, int64_t sorted_rows, int width, int ff,
                              int top, float weight, const float* pair_weight, int act_dtype, void* stream);
@@ -292,11 +300,12 @@ int swm_group_norm_add(float* residual, const void* y1, int64_t y1_stride, float
 
 /* The short causal convolution of swm_short_conv with the types and the form named: x of x_dtype, out of out_dtype
  * [rows, channels]; out = act(conv(x) + (residual != 0 ? x : 0)), act = silu when silu != 0.  The state holds the last
- * num_taps - 1 inputs in fp32; swm_short_conv_advance (with x's dtype) moves it on. */
+ * num_taps - 1 inputs in fp32; advance != 0: the same launch moves it past the step's tokens (else
+ * swm_short_conv_advance with x's dtype does). */
 int swm_causal_conv(void* out, int out_dtype, const void* x, int x_dtype, int64_t x_stride, const float* taps,
-                    const float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
+                    float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
                     const int32_t* state_slot, int64_t rows, int channels, int num_taps, int silu, int residual,
-                    void* stream);
+                    int advance, void* stream);
 
 /* swm_channel_delta with ONE decay per head: g = exp(-exp(a_log[head]) * softplus(decay_pre[t, head] + dt_bias[head])),
  * decay_pre act_dtype [rows, heads] (row stride decay_stride), dt_bias fp32 [heads].  Workspace as swm_channel_delta. */

@@ -297,7 +297,7 @@ def test_delta_rule_with_one_decay_per_head(H, G, d, dv, taps, dtype):
             x = torch.cat([proj[s][lo:lo + n] for s, lo, n, _ in step]).to(DEV)
             batch = ragged([(lo, n, slot, []) for _, lo, n, slot in step], width=1)
             qkv = torch.empty(x.shape[0], c, dtype=torch.float32, device=DEV)
-            ops().short_conv(qkv, x[:, :c], conv_w.to(DEV), conv_state, batch)
+            ops().causal_conv(qkv, x[:, :c], conv_w.to(DEV), conv_state, batch, silu=True, residual=False)
             o = torch.empty(x.shape[0], H * dv, dtype=torch.float32, device=DEV)
             ops().gated_delta(o, qkv, x[:, c:c + H], x[:, c + H:], dt_bias.to(DEV), a_log.to(DEV), rule_state, batch, H, G, d, dv)
             at = 0
@@ -398,8 +398,20 @@ def _cfg_c():
     return bu.config(layers, mlps, vocab=61, width=40, groups=5, taps=4)
 
 
-_CASES = {"a": (_cfg_a, 11), "b": (_cfg_b, 12), "c": (_cfg_c, 13)}
+def _cfg_d():
+    """The layers of ``a`` with routers that choose ALL their experts: nothing discrete is left, so bf16 runs can be
+    held against the plain statement position by position (a close call of a router that falls the other way in bf16
+    moves a position, and through the recurrent states the ones after it, by far more than rounding does)."""
+    cfg = _cfg_a()
+    for layer, size in zip(cfg["layers"], [(4, 20), (3, 16), None, (4, 24), (2, 8)]):
+        if layer["mlp"] is not None:
+            layer["mlp"] = bu.moe(size[0], size[0], size[1], 1, 1, 1.0)
+    return cfg
+
+
+_CASES = {"a": (_cfg_a, 11), "b": (_cfg_b, 12), "c": (_cfg_c, 13), "d": (_cfg_d, 14)}
 FP32_TOL = 2e-4
+BF16_TOL = 0.15         # five layers of ten normed sublayers: the worst position of a bf16 run stands near 0.10
 
 
 @pytest.fixture(scope="module")
@@ -481,7 +493,7 @@ def test_portions_of_prompts(models, engines, name, portions):
 
 
 @pytest.mark.parametrize("name,dtype,tol", [("a", "float32", FP32_TOL), ("b", "float32", FP32_TOL), ("c", "float32", FP32_TOL),
-                                            ("a", "bfloat16", 0.08)])
+                                            ("d", "bfloat16", BF16_TOL)])
 def test_mixed_batches_reuse_pages_and_slots(models, engines, name, dtype, tol):
     """Six unequal requests over three state slots and a pool of 9 pages: portions beside single tokens, requests
     that sit out steps, pages and slots handed on as requests end.  Every request must come out as it does alone."""
@@ -513,22 +525,23 @@ def test_mixed_batches_reuse_pages_and_slots(models, engines, name, dtype, tol):
             step.pop(rnd.choice(sorted(step)))                  # somebody sits this step out
         rp.step(step)
     for rid in reqs:
-        if dtype == "bfloat16":
-            assert bu.share_within(rp.result(rid), m.want[rid], tol) >= 0.8, rid
-        else:
-            assert bu.row_error(rp.result(rid), m.want[rid]) < tol, rid
+        assert bu.row_error(rp.result(rid), m.want[rid]) < tol, rid
     assert engine.scheduler.block_manager.get_num_free_gpu_blocks() == free_before
     assert engine.scheduler.state_slots.num_free() == 3
 
 
 def test_bfloat16_is_close_and_does_not_depend_on_the_cut(models, engines):
-    m = models["a"]
+    m = models["d"]
     toks = m.reqs["r0"]
-    whole = bu.Replayer(engines("a", "bfloat16"), {"r0": toks}).run_alone("r0", [len(toks)])
-    cut = bu.Replayer(engines("a", "bfloat16"), {"r0": toks}).run_alone("r0", [2, 3, 16, 1, 1, 30, 17])
-    assert bu.share_within(whole, m.want["r0"], 0.08) >= 0.8
-    assert bu.share_within(cut, m.want["r0"], 0.08) >= 0.8
-    assert bu.share_within(cut, whole, 0.05) >= 0.9
+    whole = bu.Replayer(engines("d", "bfloat16"), {"r0": toks}).run_alone("r0", [len(toks)])
+    cut = bu.Replayer(engines("d", "bfloat16"), {"r0": toks}).run_alone("r0", [2, 3, 16, 1, 1, 30, 17])
+    assert bu.row_error(whole, m.want["r0"]) < BF16_TOL
+    assert bu.row_error(cut, m.want["r0"]) < BF16_TOL
+    assert bu.row_error(cut, whole) < 0.05
+    # with routers that choose (model a) most positions still agree; the others follow a close call
+    m = models["a"]
+    whole = bu.Replayer(engines("a", "bfloat16"), {"r0": m.reqs["r0"]}).run_alone("r0", [len(m.reqs["r0"])])
+    assert bu.share_within(whole, m.want["r0"], BF16_TOL) >= 0.8
 
 
 @pytest.mark.parametrize("name", sorted(_CASES))

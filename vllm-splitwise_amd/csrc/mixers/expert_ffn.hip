@@ -24,6 +24,18 @@ __device__ __forceinline__ float expert_act(float z, int activation) {
   return gelu_erf(z);
 }
 
+// A gated hidden layer with limits, fused into the up-projection: an expert's matrix then holds, per run of 16 hidden
+// channels, the 16 gate rows followed by the 16 up rows (a last, shorter run is padded with zero rows), so that a tile
+// of 64 output columns holds gate and up products of the same 32 channels:  g = min(gate, limit),
+// u = clamp(up, -limit, limit);  hidden = g * sigmoid(alpha * g) * (u + shift).
+struct GluParams {
+  float alpha, limit, shift;
+};
+__device__ __forceinline__ float clamped_glu(float gate, float up, const GluParams& p) {
+  const float g = fminf(gate, p.limit), u = fminf(fmaxf(up, -p.limit), p.limit);
+  return g * sigmoidf_(p.alpha * g) * (u + p.shift);
+}
+
 // -> expert and first sorted row of this workgroup's tile of `tm` rows, rows in it (0: nothing to do)
 __device__ __forceinline__ int find_tile(const int32_t* __restrict__ expert_start, int num_experts, int tile,
                                          int* expert, int* row0, int tm = TM) {
@@ -86,7 +98,7 @@ template <typename T>
 __global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_kernel(
     void* __restrict__ hidden, const void* __restrict__ x, const void* __restrict__ up,
     const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
-    int top, int activation) {
+    int top, int activation, int up_rows, GluParams glu) {
   __shared__ float As[TM][TK + 1];
   __shared__ float Bs[TN][TK + 1];
   int e, row0;
@@ -94,13 +106,22 @@ __global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_kernel(
   if (rows == 0) return;
   const int n0 = blockIdx.y * TN;
   float acc[2][4];
-  tile_gemm<T>(acc, x, [&](int r) { return (int64_t)(order[row0 + r] / top); }, rows, up, (int64_t)e * ff * width, n0, ff,
-               width, As, Bs);
+  tile_gemm<T>(acc, x, [&](int r) { return (int64_t)(order[row0 + r] / top); }, rows, up, (int64_t)e * up_rows * width, n0,
+               up_rows, width, As, Bs);
   const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int r = 2 * ty + i;
     if (r >= rows) continue;
+    if (activation == SWM_ACT_CLAMPED_GLU) {
+      // columns tx + 16 j of the tile: j = 0, 2 are gate products, j = 1, 3 the up products of the same channels
+#pragma unroll
+      for (int j = 0; j < 4; j += 2) {
+        const int ch = (n0 / 32 + j / 2) * 16 + tx;
+        if (ch < ff) st<T>(hidden, (int64_t)(row0 + r) * ff + ch, clamped_glu(acc[i][j], acc[i][j + 1], glu));
+      }
+      continue;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx + 16 * j;
@@ -194,7 +215,7 @@ __device__ __forceinline__ void for_each_acc(const f32x16& acc, F&& f) {
 __global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_mfma_kernel(
     uint16_t* __restrict__ hidden, const uint16_t* __restrict__ x, const uint16_t* __restrict__ up,
     const int32_t* __restrict__ order, const int32_t* __restrict__ expert_start, int num_experts, int width, int ff,
-    int top, int activation) {
+    int top, int activation, int up_rows, GluParams glu) {
   __shared__ __attribute__((aligned(16))) uint16_t As[MM][MK + MPAD];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[MN][MK + MPAD];
   int e, row0;
@@ -202,8 +223,19 @@ __global__ __launch_bounds__(kFfnThreads) void expert_up_gelu_mfma_kernel(
   if (rows == 0) return;
   const int n0 = blockIdx.y * MN;
   f32x16 acc;
-  tile_gemm_mfma(acc, x, [&](int r) { return (int64_t)(order[row0 + r] / top); }, rows, up, (int64_t)e * ff * width, n0,
-                 ff, width, As, Bs);
+  tile_gemm_mfma(acc, x, [&](int r) { return (int64_t)(order[row0 + r] / top); }, rows, up, (int64_t)e * up_rows * width,
+                 n0, up_rows, width, As, Bs);
+  if (activation == SWM_ACT_CLAMPED_GLU) {
+    // a lane's column c of the tile: c % 32 < 16 is the gate product of channel (n0 + c) / 32 * 16 + c % 16, and lane
+    // + 16 holds the up product of the same channel and rows
+    for_each_acc(acc, [&](int r, int c, float v) {
+      const float other = __shfl_xor(v, 16, 64);
+      const int ch = (n0 + c) / 32 * 16 + c % 16;
+      if ((c & 16) == 0 && r < rows && ch < ff)
+        hidden[(int64_t)(row0 + r) * ff + ch] = sw::float_to_bf16_bits(clamped_glu(v, other, glu));
+    });
+    return;
+  }
   for_each_acc(acc, [&](int r, int c, float v) {
     if (r < rows && n0 + c < ff) hidden[(int64_t)(row0 + r) * ff + n0 + c] = sw::float_to_bf16_bits(expert_act(v, activation));
   });
@@ -247,24 +279,34 @@ int swm_expert_up_gelu(void* hidden, const void* x, const void* up, const int32_
 int swm_expert_up(void* hidden, const void* x, const void* up, const int32_t* order, const int32_t* expert_start,
                   int num_experts, int64_t sorted_rows, int width, int ff, int top, int activation, int act_dtype,
                   void* stream) {
+  return swm_expert_up_as(hidden, x, up, order, expert_start, num_experts, sorted_rows, width, ff, top, activation, 1.0f,
+                          INFINITY, 0.0f, act_dtype, stream);
+}
+
+int swm_expert_up_as(void* hidden, const void* x, const void* up, const int32_t* order, const int32_t* expert_start,
+                     int num_experts, int64_t sorted_rows, int width, int ff, int top, int activation, float glu_alpha,
+                     float glu_limit, float glu_shift, int act_dtype, void* stream) {
   using namespace swm;
   if (sorted_rows == 0) return SW_OK;
-  SW_CHECK_ARG(activation == SWM_ACT_GELU || activation == SWM_ACT_RELU2 || activation == SWM_ACT_NONE,
+  const bool gated = activation == SWM_ACT_CLAMPED_GLU;
+  const int up_rows = gated ? 32 * ((ff + 15) / 16) : ff;     // runs of 16 gate rows + 16 up rows
+  const GluParams glu{glu_alpha, glu_limit, glu_shift};
+  SW_CHECK_ARG(activation == SWM_ACT_GELU || activation == SWM_ACT_RELU2 || activation == SWM_ACT_NONE || gated,
                "expert_up: unknown activation %d", activation);
   SW_CHECK_ARG(act_ok(act_dtype), "expert_up_gelu: unsupported dtype %d", act_dtype);
   SW_CHECK_ARG(num_experts > 0 && width > 0 && ff > 0 && top > 0 && sorted_rows < (1ll << 30), "expert_up_gelu: bad shape");
   if (act_dtype == SW_BF16 && width % 8 == 0) {
-    const dim3 mgrid((unsigned)((sorted_rows + MM - 1) / MM + num_experts), (unsigned)((ff + MN - 1) / MN));
+    const dim3 mgrid((unsigned)((sorted_rows + MM - 1) / MM + num_experts), (unsigned)((up_rows + MN - 1) / MN));
     hipLaunchKernelGGL(expert_up_gelu_mfma_kernel, mgrid, dim3(kFfnThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<uint16_t*>(hidden), static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(up),
-                       order, expert_start, num_experts, width, ff, top, activation);
+                       order, expert_start, num_experts, width, ff, top, activation, up_rows, glu);
     SW_CHECK_LAUNCH();
     return SW_OK;
   }
-  const dim3 grid((unsigned)((sorted_rows + TM - 1) / TM + num_experts), (unsigned)((ff + TN - 1) / TN));
+  const dim3 grid((unsigned)((sorted_rows + TM - 1) / TM + num_experts), (unsigned)((up_rows + TN - 1) / TN));
   SWM_DISPATCH_ACT(act_dtype, hipLaunchKernelGGL(expert_up_gelu_kernel<T>, grid, dim3(kFfnThreads), 0,
                                                  static_cast<hipStream_t>(stream), hidden, x, up, order, expert_start,
-                                                 num_experts, width, ff, top, activation););
+                                                 num_experts, width, ff, top, activation, up_rows, glu););
   SW_CHECK_LAUNCH();
   return SW_OK;
 }

@@ -122,36 +122,59 @@ constexpr int kMaxTaps = 16;
 
 // TX: type of the inputs x, TO: type of the outputs.  silu: the activation after the sum; residual: the input
 // itself is added to its convolution (out = x + conv(x)).
+// advance: the launch also moves the state past the step's tokens.  Only a sequence's first num_taps - 1 rows read
+// the state, so the workgroup of the FIRST row works all of them out (the workgroups of the others leave at once) and
+// then writes the new state; a thread owns its channel in both, so nothing is read after it was overwritten.
 template <typename TX, typename TO>
 __global__ __launch_bounds__(kRowThreads) void short_conv_kernel(
     void* __restrict__ out, const void* __restrict__ x, int64_t x_stride, const float* __restrict__ taps,
-    const float* __restrict__ state, const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
+    float* __restrict__ state, const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ token_seq, const int32_t* __restrict__ state_slot, int channels, int num_taps, int silu,
-    int residual) {
-  const int64_t t = blockIdx.x;
+    int residual, int advance) {
+  const int64_t t0 = blockIdx.x;
   const int c = blockIdx.y * kRowThreads + threadIdx.x;
-  if (c >= channels) return;
-  const int s = token_seq[t];
-  const int first = q_start[s];
-  const bool carried = ctx_len[s] > 0;
-  const float* carry = state + (int64_t)state_slot[s] * (num_taps - 1) * channels;
-  float acc = 0.0f;
-  for (int j = 0; j < num_taps; ++j) {
-    const int back = num_taps - 1 - j;                  // tokens before the current one
-    const int64_t src = t - back;
-    float xv;
-    if (src >= first) {
-      xv = ld<TX>(x, src * x_stride + c);
-    } else if (carried) {
-      // the input `first - src` tokens before this step's first one: the state's row (num_taps-1) - that
-      xv = carry[(int64_t)(num_taps - 1 - (first - (int)src)) * channels + c];
-    } else {
-      xv = 0.0f;
-    }
-    acc += taps[(int64_t)c * num_taps + j] * xv;
+  const int s = token_seq[t0];
+  const int first = q_start[s], n = q_start[s + 1] - first, keep = num_taps - 1;
+  const int rel = (int)t0 - first;
+  int count = 1;
+  if (advance && keep > 0) {
+    if (rel > 0 && rel < keep) return;                  // the whole workgroup: the first row's workgroup does this row
+    if (rel == 0) count = min(keep, n);
   }
-  if (residual) acc += ld<TX>(x, t * x_stride + c);
-  st<TO>(out, t * (int64_t)channels + c, silu ? acc * sigmoidf_(acc) : acc);
+  if (c >= channels) return;
+  const bool carried = ctx_len[s] > 0;
+  float* carry = state + (int64_t)state_slot[s] * keep * channels;
+  for (int64_t t = t0; t < t0 + count; ++t) {
+    float acc = 0.0f;
+    for (int j = 0; j < num_taps; ++j) {
+      const int back = num_taps - 1 - j;                // tokens before the current one
+      const int64_t src = t - back;
+      float xv;
+      if (src >= first) {
+        xv = ld<TX>(x, src * x_stride + c);
+      } else if (carried) {
+        // the input `first - src` tokens before this step's first one: the state's row (num_taps-1) - that
+        xv = carry[(int64_t)(num_taps - 1 - (first - (int)src)) * channels + c];
+      } else {
+        xv = 0.0f;
+      }
+      acc += taps[(int64_t)c * num_taps + j] * xv;
+    }
+    if (residual) acc += ld<TX>(x, t * x_stride + c);
+    st<TO>(out, t * (int64_t)channels + c, silu ? acc * sigmoidf_(acc) : acc);
+  }
+  if (!advance || keep == 0 || rel != 0) return;
+  float fresh[kMaxTaps];
+  for (int p = 0; p < keep; ++p) {
+    // new row p holds the input (keep - p) tokens before the END of this step
+    const int off = n - (keep - p);                     // index among this step's tokens; < 0: before them
+    float v;
+    if (off >= 0) v = ld<TX>(x, (int64_t)(first + off) * x_stride + c);
+    else if (carried && keep + off >= 0) v = carry[(int64_t)(keep + off) * channels + c];
+    else v = 0.0f;
+    fresh[p] = v;
+  }
+  for (int p = 0; p < keep; ++p) carry[(int64_t)p * channels + c] = fresh[p];
 }
 
 // one thread per (sequence, channel): reads what it needs of the old state, then writes the new one
@@ -263,14 +286,14 @@ int swm_short_conv(float* out, const void* x, int64_t x_stride, const float* tap
                    const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
                    const int32_t* state_slot, int64_t rows, int channels, int num_taps, int act_dtype,
                    void* stream) {
-  return swm_causal_conv(out, SW_F32, x, act_dtype, x_stride, taps, state, q_start, ctx_len, token_seq, state_slot, rows,
-                         channels, num_taps, 1, 0, stream);
+  return swm_causal_conv(out, SW_F32, x, act_dtype, x_stride, taps, const_cast<float*>(state), q_start, ctx_len, token_seq,
+                         state_slot, rows, channels, num_taps, 1, 0, 0, stream);
 }
 
 int swm_causal_conv(void* out, int out_dtype, const void* x, int x_dtype, int64_t x_stride, const float* taps,
-                    const float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
+                    float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* token_seq,
                     const int32_t* state_slot, int64_t rows, int channels, int num_taps, int silu, int residual,
-                    void* stream) {
+                    int advance, void* stream) {
   using namespace swm;
   if (rows == 0) return SW_OK;
   SW_CHECK_ARG(act_ok(x_dtype) && act_ok(out_dtype), "causal_conv: unsupported dtype %d / %d", x_dtype, out_dtype);
@@ -280,7 +303,7 @@ int swm_causal_conv(void* out, int out_dtype, const void* x, int x_dtype, int64_
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define SWM_CONV_LAUNCH(TX, TO)                                                                                       \
   hipLaunchKernelGGL((short_conv_kernel<TX, TO>), grid, dim3(kRowThreads), 0, s, out, x, x_stride, taps, state,       \
-                     q_start, ctx_len, token_seq, state_slot, channels, num_taps, silu, residual)
+                     q_start, ctx_len, token_seq, state_slot, channels, num_taps, silu, residual, advance)
   if (x_dtype == SW_F32) {
     if (out_dtype == SW_F32) SWM_CONV_LAUNCH(float, float); else SWM_CONV_LAUNCH(float, sw::bf16_t);
   } else {

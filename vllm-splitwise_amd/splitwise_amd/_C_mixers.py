@@ -18,7 +18,7 @@ import torch
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_PKG_DIR, "libsplitwise_mixers.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 SW_F32, SW_BF16 = 0, 2
 _ACT = {torch.float32: SW_F32, torch.bfloat16: SW_BF16}
@@ -57,14 +57,15 @@ _SIGNATURES = {
     "swm_gla": [_p, _p, _p, _p, _l, _p, _l, _p, _f, _f, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
     "swm_lightning": [_p, _p, _p, _p, _l, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
     "swm_group_norm_add": [_p, _p, _l, _f, _p, _l, _f, _i, _p, _p, _p, _p, _i, _i, _f, _l, _i, _p],
-    "swm_causal_conv": [_p, _i, _p, _i, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _p],
+    "swm_causal_conv": [_p, _i, _p, _i, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
     "swm_gated_delta": [_p, _p, _p, _l, _p, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
     "swm_norm_rope_cache": [_p, _p, _p, _p, _l, _p, _p, _f, _p, _p, _i, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
     "swm_sigmoid_attention": [_p, _p, _p, _p, _p, _l, _p, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p,
                               _i, _p],
     "swm_group_router_as": [_p, _p, _p, _p, _l, _i, _i, _i, _i, _f, _i, _i, _i, _p],
+    "swm_expert_up_as": [_p, _p, _p, _p, _p, _i, _l, _i, _i, _i, _i, _f, _f, _f, _i, _p],
 }
-ACT_GELU, ACT_RELU2, ACT_NONE = 0, 1, 2
+ACT_GELU, ACT_RELU2, ACT_NONE, ACT_CLAMPED_GLU = 0, 1, 2, 3
 
 _lib = None
 
@@ -301,7 +302,7 @@ def causal_conv(out: torch.Tensor, x: torch.Tensor, taps: torch.Tensor, state: t
                 silu: bool = False, residual: bool = True) -> None:
     """out [rows, channels] (any activation dtype) = act(conv(x) + x) (``residual``) or act(conv(x)), act = silu or
     none; x: a 2-D view, fp32 or bf16; the state [slots, taps - 1, channels] (fp32: the sequence's last inputs) is read
-    and then moved past the step's tokens."""
+    and moved past the step's tokens in the same launch."""
     _dev(out, x, taps, state)
     _f32c(taps, "taps")
     _f32c(state, "state")
@@ -316,10 +317,7 @@ def causal_conv(out: torch.Tensor, x: torch.Tensor, taps: torch.Tensor, state: t
         _check(lib.swm_causal_conv(out.data_ptr(), _act(out), x.data_ptr(), _act(x), stride, taps.data_ptr(),
                                    state.data_ptr(), batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
                                    batch.token_seq.data_ptr(), batch.state_slot.data_ptr(), rows, channels, k,
-                                   1 if silu else 0, 1 if residual else 0, _stream(x)))
-        _check(lib.swm_short_conv_advance(state.data_ptr(), x.data_ptr(), stride, batch.q_start.data_ptr(),
-                                          batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), n, channels, k,
-                                          _act(x), _stream(x)))
+                                   1 if silu else 0, 1 if residual else 0, 1, _stream(x)))
 
 
 def gated_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, decay_pre: torch.Tensor,
@@ -417,19 +415,22 @@ def expert_ffn(out: torch.Tensor, x: torch.Tensor, up: torch.Tensor, down: torch
     """out (fp32 [rows, width], zeroed by the caller) += weight * sum over each row's experts of
     pair_weight[row, choice] * down[e] act(up[e] x[row]); ``order`` / ``expert_start``: the (row, choice) pairs
     sorted by expert and every expert's first sorted pair; ``activation``: ACT_GELU (exact gelu) or ACT_RELU2;
-    ``pair_weight`` fp32 [rows, top] (None: all 1).  ``glu`` = (alpha, limit, shift): a gated hidden layer -- ``up``
-    holds every expert's gate rows and then its up rows ([experts, 2 * ff, width]) and the hidden layer is
-    g sigmoid(alpha g) (u + shift) with g = min(gate x, limit), u = clamp(up x, -limit, limit)."""
+    ``pair_weight`` fp32 [rows, top] (None: all 1).  ``glu`` = (alpha, limit, shift): a gated hidden layer,
+    g sigmoid(alpha g) (u + shift) with g = min(gate x, limit), u = clamp(up x, -limit, limit), worked out in the
+    up-projection's epilogue -- ``up`` then holds gate and up rows in runs of 16 (``glu_rows``)."""
     _dev(out, x, up, down, order, expert_start, pair_weight)
     _f32c(out, "out")
     rows, width = x.shape
     experts, ff = up.shape[0], up.shape[1]
+    alpha, limit, shift = 1.0, float("inf"), 0.0
     if glu is not None:
-        _need(ff % 2 == 0, "expert_ffn: a gated hidden layer has gate and up rows")
-        activation = ACT_NONE
+        ff = down.shape[2]
+        _need(up.shape[1] == 32 * (-(-ff // 16)), "expert_ffn: a gated hidden layer takes gate and up rows in runs of 16")
+        activation = ACT_CLAMPED_GLU
+        alpha, limit, shift = (float(v) for v in glu)
     _need(x.is_contiguous() and up.is_contiguous() and down.is_contiguous() and up.dtype == x.dtype == down.dtype
-          and up.shape == (experts, ff, width) and out.shape == (rows, width)
-          and down.shape == (experts, width, ff // 2 if glu is not None else ff)
+          and up.shape[::2] == (experts, width) and (glu is not None or up.shape[1] == ff) and out.shape == (rows, width)
+          and down.shape == (experts, width, ff)
           and order.dtype == torch.int32 and order.numel() == rows * top and order.is_contiguous()
           and expert_start.dtype == torch.int32 and expert_start.numel() == experts + 1
           and expert_start.is_contiguous(), "expert_ffn: shapes")
@@ -440,19 +441,26 @@ def expert_ffn(out: torch.Tensor, x: torch.Tensor, up: torch.Tensor, down: torch
     hidden = torch.empty(pairs, ff, dtype=x.dtype, device=x.device)
     with _on_device_of(x):
         lib = load_library()
-        _check(lib.swm_expert_up(hidden.data_ptr(), x.data_ptr(), up.data_ptr(), order.data_ptr(),
-                                 expert_start.data_ptr(), experts, pairs, width, ff, top, activation, _act(x),
-                                 _stream(x)))
-        if glu is not None:
-            ff //= 2
-            gated = torch.empty(pairs, ff, dtype=x.dtype, device=x.device)
-            _check(lib.swm_clamped_glu(gated.data_ptr(), hidden.data_ptr(), 2 * ff, pairs, ff, float(glu[0]),
-                                       float(glu[1]), float(glu[2]), _act(x), _stream(x)))
-            hidden = gated
+        _check(lib.swm_expert_up_as(hidden.data_ptr(), x.data_ptr(), up.data_ptr(), order.data_ptr(),
+                                    expert_start.data_ptr(), experts, pairs, width, ff, top, activation, alpha, limit,
+                                    shift, _act(x), _stream(x)))
         _check(lib.swm_expert_down_weighted(out.data_ptr(), hidden.data_ptr(), down.data_ptr(), order.data_ptr(),
                                             expert_start.data_ptr(), experts, pairs, width, ff, top, weight,
                                             None if pair_weight is None else pair_weight.data_ptr(), _act(x),
                                             _stream(x)))
+
+
+def glu_rows(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """gate, up [..., ff, width] -> [..., 32 * ceil(ff / 16), width]: per run of 16 hidden channels the 16 gate rows, then
+    the 16 up rows (a shorter last run padded with zero rows): what ``expert_ffn(glu=...)`` takes as ``up``."""
+    ff, width = gate.shape[-2:]
+    runs = -(-ff // 16)
+    pad = runs * 16 - ff
+    if pad:
+        zeros = gate.new_zeros(gate.shape[:-2] + (pad, width))
+        gate, up = torch.cat([gate, zeros], -2), torch.cat([up, zeros], -2)
+    both = torch.stack([gate.unflatten(-2, (runs, 16)), up.unflatten(-2, (runs, 16))], -3)     # [..., runs, 2, 16, width]
+    return both.flatten(-4, -2).contiguous()
 
 
 def _opt_ptr(t: Optional[torch.Tensor]):
@@ -838,5 +846,5 @@ ops = SimpleNamespace(expert_ffn=expert_ffn, ACT_GELU=ACT_GELU, ACT_RELU2=ACT_RE
     general_delta=general_delta, head_norm_gate=head_norm_gate, stream_add_norm=stream_add_norm,
     clamped_glu=clamped_glu, relu2=relu2, rope_cache=rope_cache, group_router=group_router, group_pairs=group_pairs,
     capped_attention=capped_attention, lightning=lightning, gated_stream_step=gated_stream_step, poly_norm=poly_norm,
-    gate_mul=gate_mul, latent_rope_cache=latent_rope_cache, gla=gla, ACT_NONE=ACT_NONE,
+    gate_mul=gate_mul, latent_rope_cache=latent_rope_cache, gla=gla, ACT_NONE=ACT_NONE, glu_rows=glu_rows,
     group_norm_add=group_norm_add, causal_conv=causal_conv, gated_delta=gated_delta)

@@ -1,4 +1,4 @@
-"""Throughput of a Nepevik (or Lapilorn, or Lalasun) stack beside a Llama stack of the same width, depth and active feed-forward size
+"""Throughput of a Nepevik (or Lapilorn, Lalasun or Bogetar) stack beside a Llama stack of the same width, depth and active feed-forward size
 (random weights), and every mixer kernel beside the like kernel of the Llama path with their distances from
 the roofline.  ``bench.py --mixers`` prints the result as one JSON line.
 
@@ -534,6 +534,148 @@ def kernel_table_lalasun(width: int = 2048, heads: int = 16, kv_heads: int = 4, 
     return rows
 
 
+@torch.inference_mode()
+def kernel_table_bogetar(width: int = 2048, heads: int = 16, kv_heads: int = 4, prefill_rows: int = 4096,
+                         decode_seqs: int = 64, decode_ctx: int = 2047, span: int = 1024, groups: int = 8, taps: int = 4,
+                         experts: int = 32, top: int = 2, ff: int = 1408) -> List[dict]:
+    """The kernels of the Bogetar layers beside their like: attention with sigmoid weights beside the same kernel with
+    a softmax (as Lapilorn runs it, same window); the rotation kernel with the per-head norm beside the plain one; the
+    delta rule with one decay per head beside Nepevik's with one per key channel; the grouped norm with its add beside
+    the fused add + RMS norm; the convolution added to a sublayer's input beside the short convolution with silu; the
+    softmax router beside the sigmoid router; experts with a gated hidden layer beside experts with relu^2."""
+    from .. import _C
+    dev, bf = torch.device("cuda"), torch.bfloat16
+    d = width // heads
+    page = 16
+    rows: List[dict] = []
+    scale = d ** -0.5
+    for phase, seqs in (("prefill", [(0, prefill_rows // 2, 0, None), (0, prefill_rows // 2, 1, None)]),
+                        ("decode", [(decode_ctx, 1, i, None) for i in range(decode_seqs)])):
+        total_pages, laid = 0, []
+        for ctx, n, slot, _ in seqs:
+            pages = -(-(ctx + n) // page)
+            laid.append((ctx, n, slot, list(range(total_pages, total_pages + pages))))
+            total_pages += pages
+        batch = _ragged(laid, dev)
+        T, B = sum(s[1] for s in laid), len(laid)
+        pairs = keys = 0
+        for c, n, _, _ in laid:
+            pairs += sum(min(i + 1, span) for i in range(c, c + n))
+            keys += c + n - max(0, (c if n == 1 else 0) - span + 1)
+        # ---------------------------------------------------------------- attention
+        kc = torch.randn(total_pages, page, kv_heads * d, device=dev).to(bf)
+        vc = torch.randn(total_pages, page, kv_heads * d, device=dev).to(bf)
+        q = torch.randn(T, heads * d, device=dev)
+        gate = torch.randn(T, heads * d, device=dev).to(bf)
+        out = torch.empty(T, heads * d, dtype=bf, device=dev)
+        bias = torch.full((heads,), -3.0, device=dev)
+        abytes = keys * kv_heads * d * 2 * 2 + T * heads * d * (4 + 2 + 2)
+        for name, kw, like in (("sigmoid attention (window %d, bias, gate)" % span, dict(score_bias=bias), ""),
+                               ("capped_attention with a softmax, same window and gate", {}, "sigmoid attention")):
+            t = _time(lambda: _C.mixer_ops.capped_attention(out, q, kc, vc, gate, batch, heads, kv_heads, d, d, scale, 0.0, span, **kw))
+            rows.append(_row(name, phase, t, abytes, 4.0 * pairs * heads * d, VALU_F32, like=like))
+        # ---------------------------------------------------------------- rotation and cache writes
+        pos = torch.cat([torch.arange(c, c + n) for c, n, _, _ in laid]).to(dev)
+        slots = torch.cat([torch.tensor([tb[p // page] * page + p % page for p in range(c, c + n)])
+                           for c, n, _, tb in laid]).to(dev)
+        proj = torch.randn(T, (heads + 2 * kv_heads) * d, device=dev).to(bf)
+        inv = torch.rand(d // 4, device=dev)
+        q32 = torch.empty(T, heads * d, device=dev)
+        wq = torch.ones(d, device=dev)
+        rbytes = T * ((heads + 2 * kv_heads) * d * 2 + heads * d * 4 + 2 * kv_heads * d * 2)
+        for name, norm, like in (("rope_cache behind a per-head norm", (wq, wq, 1e-6), ""), ("rope_cache", (), "rope_cache + norm")):
+            t = _time(lambda: _C.mixer_ops.rope_cache(q32, proj[:, :heads * d], proj[:, heads * d:(heads + kv_heads) * d],
+                                                      proj[:, (heads + kv_heads) * d:], pos, inv, heads, kv_heads, d, d, kc,
+                                                      vc, slots, True, *norm))
+            rows.append(_row(name, phase, t, rbytes, (10.0 if norm else 6.0) * T * heads * d, VALU_F32, like=like))
+        # ---------------------------------------------------------------- delta rules
+        lbatch = _ragged([(c, n, i, []) for i, (c, n, _, _) in enumerate(laid)], dev)
+        G = heads // 2
+        c_ = 2 * G * d + heads * d
+        dproj = torch.randn(T, c_ + 2 * heads, device=dev).to(bf)
+        ctaps = torch.randn(c_, taps, device=dev) * 0.3
+        cstate = torch.zeros(max(B, 2), taps - 1, c_, device=dev)
+        rstate = torch.zeros(max(B, 2), heads, d, d, device=dev)
+        qkv = torch.empty(T, c_, device=dev)
+        o = torch.empty(T, heads * d, device=dev)
+        zero_h, zero_hd = torch.zeros(heads, device=dev), torch.zeros(heads * d, device=dev)
+        dpre = torch.randn(T, heads * d, device=dev).to(bf)
+        t = _time(lambda: _C.mixer_ops.short_conv(qkv, dproj[:, :c_], ctaps, cstate, lbatch))
+        rows.append(_row("short_conv + state advance (q | k | v, silu)", phase, t, T * c_ * (2 + 4), 2.0 * taps * T * c_, VALU_F32))
+        dflops = T * heads * 6.0 * d * d
+        dbytes = T * (c_ * 4 + heads * d * 4) + 2 * B * heads * d * d * 4
+        t = _time(lambda: _C.mixer_ops.gated_delta(o, qkv, dproj[:, c_:c_ + heads], dproj[:, c_ + heads:], zero_h, zero_h, rstate,
+                                                   lbatch, heads, G, d, d))
+        rows.append(_row("gated_delta (one decay per head; prologue + recurrence)", phase, t, dbytes, dflops, VALU_F32))
+        t = _time(lambda: _C.mixer_ops.channel_delta(o, qkv, dproj[:, c_:c_ + heads], dpre, zero_hd, zero_h, rstate, lbatch, heads,
+                                                     G, d, d))
+        rows.append(_row("Nepevik channel_delta (a decay per key channel), same sizes", phase, t, dbytes + T * heads * d * 2, dflops,
+                         VALU_F32, like="gated_delta"))
+        # ---------------------------------------------------------------- gated linear attention at this design's sizes
+        rh, dk = heads // 4, d // 2
+        gproj = torch.randn(T, rh * (2 * dk + d), device=dev).to(bf)
+        zpre = torch.randn(T, rh * dk, device=dev).to(bf)
+        zbias = torch.full((rh * dk,), 2.0, device=dev)
+        gstate = torch.zeros(max(B, 2), rh, dk, d, device=dev)
+        go = torch.empty(T, rh * d, device=dev)
+        t = _time(lambda: _C.mixer_ops.gla(go, gproj[:, :rh * dk], gproj[:, rh * dk:2 * rh * dk], gproj[:, 2 * rh * dk:], zpre, zbias,
+                                           16.0, dk ** -0.5, gstate, lbatch, rh, dk, d))
+        rows.append(_row("gla (%d heads beside the attention)" % rh, phase, t,
+                         T * rh * ((3 * dk + d) * 2 + d * 4) + 2 * B * rh * dk * d * 4,
+                         T * rh * (2.0 * 32 * dk + 2.0 * 32 * d + 4.0 * dk * d), VALU_F32))
+        # ---------------------------------------------------------------- norms and the convolution on a sublayer's input
+        stream = torch.randn(T, width, device=dev)
+        y = torch.randn(T, 2 * width, device=dev).to(bf)
+        y32 = torch.randn(T, width, device=dev)
+        wn = torch.ones(width, device=dev)
+        h32 = torch.empty(T, width, device=dev)
+        t = _time(lambda: _C.mixer_ops.group_norm_add(stream, groups, 1e-6, y[:, :width], wn, wn, None, 1.0, 1.0, wn, h32))
+        rows.append(_row("group_norm_add (one addend, %d groups, fp32 norm out)" % groups, phase, t, T * width * (4 + 4 + 2 + 4),
+                         12.0 * T * width, VALU_F32))
+        t = _time(lambda: _C.mixer_ops.group_norm_add(stream, groups, 1e-6, y[:, :width], wn, wn, y[:, width:], 0.8, 0.5, wn, h32))
+        rows.append(_row("group_norm_add (two addends)", phase, t, T * width * (4 + 4 + 2 + 2 + 4), 14.0 * T * width, VALU_F32))
+        t = _time(lambda: _C.mixer_ops.group_norm_add(stream, groups, 1e-6, y32, wn, wn, None, 1.0, 1.0, wn, h32))
+        rows.append(_row("group_norm_add (fp32 addend: the experts' sum)", phase, t, T * width * (4 + 4 + 4 + 4), 12.0 * T * width,
+                         VALU_F32))
+        hout = torch.empty(T, width, dtype=bf, device=dev)
+        t2 = _time(lambda: _C.mixer_ops.stream_add_norm(stream, wn, 1.0, 1e-6, hout, y[:, :width], y[:, width:], None))
+        rows.append(_row("Lapilorn stream_add_norm (two addends)", phase, t2, T * width * (4 + 4 + 2 + 2 + 2), 6.0 * T * width, VALU_F32,
+                         like="group_norm_add"))
+        wtaps = torch.randn(width, taps, device=dev) * 0.3
+        wstate = torch.zeros(max(B, 2), taps - 1, width, device=dev)
+        t = _time(lambda: _C.mixer_ops.causal_conv(hout, h32, wtaps, wstate, lbatch))
+        rows.append(_row("causal_conv added to its input + state advance (fp32 in)", phase, t, T * width * (4 + 2), 2.0 * taps * T * width,
+                         VALU_F32, like="short_conv"))
+        # ---------------------------------------------------------------- router and experts
+        logits = torch.randn(T, experts, device=dev)
+        t = _time(lambda: _C.mixer_ops.group_router(logits, None, top, 4, 2, 1.0, True, True, False))
+        rows.append(_row("group_router (softmax, best-of-group, weights as they are)", phase, t, T * experts * 4 + T * top * 8,
+                         8.0 * T * experts, VALU_F32))
+        t2 = _time(lambda: _C.mixer_ops.group_router(logits, None, top, 4, 2, 1.0))
+        rows.append(_row("Lapilorn group_router (sigmoid)", phase, t2, T * experts * 4 + T * top * 8, 8.0 * T * experts, VALU_F32,
+                         like="group_router"))
+        chosen, weights = _C.mixer_ops.group_router(logits, None, top, 4, 2, 1.0, True, True, False)
+        order, start = _C.mixer_ops.group_pairs(chosen, experts)
+        x = torch.randn(T, width, device=dev).to(bf)
+        up_glu = (torch.randn(experts, 32 * (-(-ff // 16)), width, device=dev) * 0.02).to(bf)
+        down = (torch.randn(experts, width, ff, device=dev) * 0.02).to(bf)
+        eo = torch.zeros(T, width, device=dev)
+        active = min(experts, T * top)
+        ebytes = active * 3 * ff * width * 2 + T * width * (2 + 4) + T * top * ff * 2 * 2
+        t = _time(lambda: _C.mixer_ops.expert_ffn(eo, x, up_glu, down, order, start, top, 1.0, pair_weight=weights,
+                                                  glu=(1.702, 7.0, 1.0)))
+        rows.append(_row("expert_ffn (gated hidden layer with limits)", phase, t, ebytes, 6.0 * T * top * ff * width, MFMA_BF16))
+        ff2 = 3 * ff // 2                                  # relu^2 experts of the same weights' size: up + down of 1.5 ff
+        up_r = (torch.randn(experts, ff2, width, device=dev) * 0.02).to(bf)
+        down_r = (torch.randn(experts, width, ff2, device=dev) * 0.02).to(bf)
+        t2 = _time(lambda: _C.mixer_ops.expert_ffn(eo, x, up_r, down_r, order, start, top, 1.0, activation=_C.mixer_ops.ACT_RELU2,
+                                                   pair_weight=weights))
+        rows.append(_row("Lapilorn expert_ffn (relu^2), same weights' size", phase, t2,
+                         active * 2 * ff2 * width * 2 + T * width * (2 + 4) + T * top * ff2 * 2 * 2, 4.0 * T * top * ff2 * width,
+                         MFMA_BF16, like="expert_ffn"))
+    return rows
+
+
 def run(sizes=("2k",), with_kernels: bool = True, family: str = "nepevik") -> dict:
     result = {"family": family, "engine": {}, "kernels": {}}
     for size in sizes:
@@ -542,6 +684,7 @@ def run(sizes=("2k",), with_kernels: bool = True, family: str = "nepevik") -> di
             pair[name] = {k: round(v, 2) for k, v in engine_throughput(f"{name}-{size}").items()}
         result["engine"][size] = pair
     if with_kernels:
-        table = {"nepevik": kernel_table, "lapilorn": kernel_table_lapilorn, "lalasun": kernel_table_lalasun}[family]
+        table = {"nepevik": kernel_table, "lapilorn": kernel_table_lapilorn, "lalasun": kernel_table_lalasun,
+                 "bogetar": kernel_table_bogetar}[family]
         result["kernels"]["2k"] = table()
     return result

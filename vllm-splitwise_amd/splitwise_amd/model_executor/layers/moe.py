@@ -98,8 +98,8 @@ class GroupRoutedExperts(nn.Module):
         # the router is fp32 whatever the model's dtype
         self.router = nn.Parameter(torch.zeros(num_experts, width, dtype=torch.float32), requires_grad=False)
         self.correction = nn.Parameter(torch.zeros(num_experts, dtype=torch.float32), requires_grad=False)
-        # a gated hidden layer: every expert's gate rows, then its up rows
-        self.up = nn.Parameter(torch.empty(num_experts, (2 if self.glu else 1) * ff, width, dtype=dtype),
+        # a gated hidden layer: gate and up rows in runs of 16, as the fused kernel reads them (``mixer_ops.glu_rows``)
+        self.up = nn.Parameter(torch.empty(num_experts, 32 * (-(-ff // 16)) if self.glu else ff, width, dtype=dtype),
                                requires_grad=False)
         self.down = nn.Parameter(torch.empty(num_experts, width, ff, dtype=dtype), requires_grad=False)
         self.shared_ff = shared_ff
@@ -131,8 +131,8 @@ class GroupRoutedExperts(nn.Module):
         if "correction" in w:
             self.correction.data.copy_(w["correction"].float())
         if self.glu:
-            self.up.data.copy_(torch.stack([torch.cat([w[f"e{e}.gate"], w[f"e{e}.up"]], 0)
-                                            for e in range(self.num_experts)]))
+            self.up.data.copy_(_C.mixer_ops.glu_rows(torch.stack([w[f"e{e}.gate"] for e in range(self.num_experts)]),
+                                                     torch.stack([w[f"e{e}.up"] for e in range(self.num_experts)])))
         else:
             self.up.data.copy_(torch.stack([w[f"e{e}.up"] for e in range(self.num_experts)]))
         self.down.data.copy_(torch.stack([w[f"e{e}.down"] for e in range(self.num_experts)]))

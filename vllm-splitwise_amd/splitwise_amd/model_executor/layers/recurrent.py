@@ -120,7 +120,7 @@ class GatedDeltaMixer(nn.Module):
         rows, c, H = h.shape[0], self.conv_channels, self.heads
         proj = self.in_proj(h)
         qkv = torch.empty(rows, c, dtype=torch.float32, device=h.device)
-        _C.mixer_ops.short_conv(qkv, proj[:, :c], self.conv_taps.data, conv_state, batch)
+        _C.mixer_ops.causal_conv(qkv, proj[:, :c], self.conv_taps.data, conv_state, batch, silu=True, residual=False)
         o = torch.empty(rows, H * self.vdim, dtype=torch.float32, device=h.device)
         _C.mixer_ops.gated_delta(o, qkv, proj[:, c:c + H], proj[:, c + H:c + 2 * H], self.dt_bias.data, self.a_log.data,
                                  rule_state, batch, H, self.kv_heads, self.dim, self.vdim)
