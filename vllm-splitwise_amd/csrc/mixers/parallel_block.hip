@@ -184,9 +184,103 @@ __global__ __launch_bounds__(kPbThreads) void rope_cache_kernel(
     st<T>(value_cache, slot * (int64_t)kv_heads * vdim + e, ld<T>(v, row + e));
 }
 
-// one wave per row: scores by the lanes, the choice by lane 0 (a few hundred LDS reads for the usual sizes)
+// The choice of one row by one wave: scores by the lanes, the choice by lane 0 (a few hundred LDS reads for the usual
+// sizes).  logits: the row's `experts` numbers (global or LDS); score, choice: LDS scratch of the wave.
 constexpr int kMaxRouterExperts = 256;
 
+__device__ __forceinline__ void router_choice(int lane, const float* __restrict__ logits, float* score, float* choice,
+                                              const float* __restrict__ correction, int experts, int top, int groups,
+                                              int keep, float scale, int softmax, int group_best_one, int normalize,
+                                              int32_t* __restrict__ chosen, float* __restrict__ weights) {
+  float top_logit = 0.0f, inv_sum = 1.0f;
+  if (softmax) {                                             // scores: the softmax over ALL experts
+    float m = -INFINITY;
+    for (int e = lane; e < experts; e += 64) m = fmaxf(m, logits[e]);
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    float sum = 0.0f;
+    for (int e = lane; e < experts; e += 64) sum += expf(logits[e] - m);
+    top_logit = m;
+    inv_sum = 1.0f / sw::wave_sum(sum);
+  }
+  for (int e = lane; e < experts; e += 64) {
+    const float z = logits[e];
+    const float s = softmax ? expf(z - top_logit) * inv_sum : sigmoidf_(z);
+    score[e] = s;
+    choice[e] = s + (correction != nullptr ? correction[e] : 0.0f);
+  }
+  __builtin_amdgcn_wave_barrier();
+  __threadfence_block();
+  // Lane l holds the candidates e = l + 64 k (and the groups g = l + 64 k); every pick is an arg-max over the wave.
+  constexpr int PER = kMaxRouterExperts / 64;
+  const float kOut = -INFINITY;
+  float cand[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) cand[k] = lane + 64 * k < experts ? choice[lane + 64 * k] : kOut;
+  if (groups > 1 && keep < groups) {
+    const int size = experts / groups;
+    // a group's score: its two largest choice scores (or its largest); the groups outside the best `keep` leave the choice
+    float gs[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int g = lane + 64 * k;
+      gs[k] = INFINITY;                                      // no such group, or one already dropped: never the worst
+      if (g < groups) {
+        float first = kOut, second = kOut;
+        for (int j = 0; j < size; ++j) {
+          const float c = choice[g * size + j];
+          if (c > first) { second = first; first = c; }
+          else if (c > second) second = c;
+        }
+        gs[k] = (size > 1 && !group_best_one) ? first + second : first;
+      }
+    }
+    for (int drop = 0; drop < groups - keep; ++drop) {
+      float lv = INFINITY;
+      int lg = -1;
+#pragma unroll
+      for (int k = 0; k < PER; ++k)                          // ties: the later group goes first
+        if (lane + 64 * k < groups && gs[k] <= lv && gs[k] != INFINITY) { lv = gs[k]; lg = lane + 64 * k; }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(lv, off, 64);
+        const int og = __shfl_xor(lg, off, 64);
+        if (og >= 0 && (lg < 0 || ov < lv || (ov == lv && og > lg))) { lv = ov; lg = og; }
+      }
+#pragma unroll
+      for (int k = 0; k < PER; ++k) {
+        if (lane + 64 * k == lg) gs[k] = INFINITY;
+        if (lane + 64 * k < experts && (lane + 64 * k) / size == lg) cand[k] = kOut;
+      }
+    }
+  }
+  float total = 0.0f;
+  for (int n = 0; n < top; ++n) {
+    float lv = kOut;
+    int le = 1 << 30;
+#pragma unroll
+    for (int k = 0; k < PER; ++k)                            // ties: the earlier expert
+      if (lane + 64 * k < experts && (cand[k] > lv || le == (1 << 30))) { lv = cand[k]; le = lane + 64 * k; }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(lv, off, 64);
+      const int oe = __shfl_xor(le, off, 64);
+      if (ov > lv || (ov == lv && oe < le)) { lv = ov; le = oe; }
+    }
+#pragma unroll
+    for (int k = 0; k < PER; ++k)
+      if (lane + 64 * k == le) cand[k] = kOut;
+    if (lane == 0) {
+      chosen[n] = le;
+      weights[n] = score[le];
+    }
+    total += score[le];
+  }
+  if (lane != 0) return;
+  const float f = normalize ? scale / (total + 1e-20f) : scale;
+  for (int n = 0; n < top; ++n) weights[n] *= f;
+}
+
+// one wave per row, logits given
 __global__ __launch_bounds__(256) void group_router_kernel(
     int32_t* __restrict__ chosen, float* __restrict__ weights, const float* __restrict__ logits,
     const float* __restrict__ correction, int64_t rows, int experts, int top, int groups, int keep, float scale,
@@ -195,68 +289,10 @@ __global__ __launch_bounds__(256) void group_router_kernel(
   __shared__ float s_choice[4][kMaxRouterExperts];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * 4 + wave;
-  const bool live = t < rows;
-  float* score = s_score[wave];
-  float* choice = s_choice[wave];
-  if (live) {
-    float top_logit = 0.0f, inv_sum = 1.0f;
-    if (softmax) {                                           // scores: the softmax over ALL experts
-      float m = -INFINITY;
-      for (int e = lane; e < experts; e += 64) m = fmaxf(m, logits[t * experts + e]);
-      for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
-      float sum = 0.0f;
-      for (int e = lane; e < experts; e += 64) sum += expf(logits[t * experts + e] - m);
-      top_logit = m;
-      inv_sum = 1.0f / sw::wave_sum(sum);
-    }
-    for (int e = lane; e < experts; e += 64) {
-      const float z = logits[t * experts + e];
-      const float s = softmax ? expf(z - top_logit) * inv_sum : sigmoidf_(z);
-      score[e] = s;
-      choice[e] = s + (correction != nullptr ? correction[e] : 0.0f);
-    }
-  }
-  __syncthreads();
-  if (!live) return;
-  if (lane != 0) return;
-  const float kOut = -INFINITY;
-  if (groups > 1 && keep < groups) {
-    const int size = experts / groups;
-    // a group's score: its two largest choice scores; the groups outside the best `keep` leave the choice
-    uint64_t dropped[kMaxRouterExperts / 64] = {};
-    for (int drop = 0; drop < groups - keep; ++drop) {
-      int worst = -1;
-      float worst_score = 0.0f;
-      for (int g = groups - 1; g >= 0; --g) {                // ties: the later group goes first
-        if ((dropped[g >> 6] >> (g & 63)) & 1ull) continue;
-        float first = kOut, second = kOut;
-        for (int j = 0; j < size; ++j) {
-          const float c = choice[g * size + j];
-          if (c > first) { second = first; first = c; }
-          else if (c > second) second = c;
-        }
-        const float gs = (size > 1 && !group_best_one) ? first + second : first;
-        if (worst < 0 || gs < worst_score) { worst = g; worst_score = gs; }
-      }
-      dropped[worst >> 6] |= 1ull << (worst & 63);
-      for (int j = 0; j < size; ++j) choice[worst * size + j] = kOut;
-    }
-  }
-  float total = 0.0f;
-  for (int n = 0; n < top; ++n) {
-    int best = 0;
-    float best_choice = choice[0];
-    for (int e = 1; e < experts; ++e)
-      if (choice[e] > best_choice) { best = e; best_choice = choice[e]; }   // ties: the earlier expert
-    choice[best] = kOut;                                    // (an expert already taken has -inf and loses every tie but the last)
-    chosen[t * top + n] = best;
-    weights[t * top + n] = score[best];
-    total += score[best];
-  }
-  const float f = normalize ? scale / (total + 1e-20f) : scale;
-  for (int n = 0; n < top; ++n) weights[t * top + n] *= f;
+  if (t >= rows) return;                                     // uniform over the wave; no workgroup barrier below
+  router_choice(lane, logits + t * experts, s_score[wave], s_choice[wave], correction, experts, top, groups, keep, scale,
+                softmax, group_best_one, normalize, chosen + t * top, weights + t * top);
 }
-
 
 // (row, choice) pairs grouped by expert in ONE launch of one workgroup: a histogram of the chosen experts in LDS, its
 // running sum = every expert's first sorted pair, then every pair takes the next place of its expert.  The order
