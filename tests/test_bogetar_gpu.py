@@ -409,7 +409,12 @@ def _cfg_d():
     return cfg
 
 
-_CASES = {"a": (_cfg_a, 11), "b": (_cfg_b, 12), "c": (_cfg_c, 13), "d": (_cfg_d, 14)}
+def _cfg_e():
+    """The least there can be: one layer without a feed-forward, convolutions of a single tap (nothing is carried)."""
+    return bu.config([bu.delta(2, 2, 8, 8, conv=1)], [None], vocab=41, width=16, groups=2, taps=1)
+
+
+_CASES = {"a": (_cfg_a, 11), "b": (_cfg_b, 12), "c": (_cfg_c, 13), "d": (_cfg_d, 14), "e": (_cfg_e, 15)}
 FP32_TOL = 2e-4
 BF16_TOL = 0.15         # five layers of ten normed sublayers: the worst position of a bf16 run stands near 0.10
 
