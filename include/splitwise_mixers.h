@@ -315,6 +315,16 @@ int swm_gated_delta(float* out, const float* qkv, const void* beta_pre, int64_t 
                     int num_seqs, int heads, int kv_heads, int dim, int vdim, float* workspace, int act_dtype,
                     void* stream);
 
+/* The same rule in chunks of 32 tokens on the matrix cores, for steps that bring long runs (any step is right, steps of
+ * few tokens per sequence are faster with swm_gated_delta): a prologue parallel over (chunk, head), then one walk over
+ * each sequence's chunks.  `workspace`: swm_gated_delta_chunked_workspace_floats() floats. */
+int64_t swm_gated_delta_chunked_workspace_floats(int64_t rows, int num_seqs, int heads, int dim, int vdim);
+int swm_gated_delta_chunked(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride,
+                            const void* decay_pre, int64_t decay_stride, const float* dt_bias, const float* a_log,
+                            float* state, const int32_t* q_start, const int32_t* ctx_len, const int32_t* state_slot,
+                            int64_t rows, int num_seqs, int heads, int kv_heads, int dim, int vdim, float* workspace,
+                            int act_dtype, void* stream);
+
 /* swm_rope_cache behind an RMS norm of every query and key head over its `dim` coordinates:
  * x / sqrt(mean(x^2) + norm_eps) * q_norm (k_norm), fp32 [dim] weights shared by the heads; q_norm NULL: no norm. */
 int swm_norm_rope_cache(float* q_out, const void* q, const void* k, const void* v, int64_t in_stride,

@@ -278,10 +278,13 @@ def test_sigmoid_weights_when_keys_are_shared_among_workgroups(cache_dtype):
 @pytest.mark.parametrize("H,G,d,dv,taps", [(3, 3, 12, 8, 4), (4, 2, 8, 20, 2), (1, 1, 64, 64, 4), (6, 1, 33, 10, 3), (2, 2, 130, 48, 5),
                                            (2, 1, 256, 16, 4)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_delta_rule_with_one_decay_per_head(H, G, d, dv, taps, dtype):
+@pytest.mark.parametrize("chunked", [None, True])
+def test_delta_rule_with_one_decay_per_head(H, G, d, dv, taps, dtype, chunked):
     """The short convolution with silu, unit queries and keys, beta, the per-head decay and the rule itself: two
     sequences interleaved over three slots that hold NaN, portions of one and two tokens, 40 tokens decoded one by
-    one; then both as whole prompts in other slots."""
+    one; then both as whole prompts in other slots.  ``chunked`` None: steps that bring 32 tokens or more of a sequence
+    go through the chunks of 32 on the matrix cores, the others token by token; True: every step goes through the
+    chunks (a decoded token is a chunk of one, runs end inside chunks, the state passes from route to route)."""
     g = torch.Generator().manual_seed(H * 100 + d)
     c = 2 * G * d + H * dv
     lens = {"a": 150, "b": 61}
@@ -299,7 +302,8 @@ def test_delta_rule_with_one_decay_per_head(H, G, d, dv, taps, dtype):
             qkv = torch.empty(x.shape[0], c, dtype=torch.float32, device=DEV)
             ops().causal_conv(qkv, x[:, :c], conv_w.to(DEV), conv_state, batch, silu=True, residual=False)
             o = torch.empty(x.shape[0], H * dv, dtype=torch.float32, device=DEV)
-            ops().gated_delta(o, qkv, x[:, c:c + H], x[:, c + H:], dt_bias.to(DEV), a_log.to(DEV), rule_state, batch, H, G, d, dv)
+            ops().gated_delta(o, qkv, x[:, c:c + H], x[:, c + H:], dt_bias.to(DEV), a_log.to(DEV), rule_state, batch, H, G, d, dv,
+                              chunked=chunked)
             at = 0
             for s, lo, n, _ in step:
                 outs[s][lo:lo + n] = o[at:at + n].cpu().double()

@@ -59,6 +59,7 @@ _SIGNATURES = {
     "swm_group_norm_add": [_p, _p, _l, _f, _p, _l, _f, _i, _p, _p, _p, _p, _i, _i, _f, _l, _i, _p],
     "swm_causal_conv": [_p, _i, _p, _i, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
     "swm_gated_delta": [_p, _p, _p, _l, _p, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
+    "swm_gated_delta_chunked": [_p, _p, _p, _l, _p, _l, _p, _p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _i, _p],
     "swm_norm_rope_cache": [_p, _p, _p, _p, _l, _p, _p, _f, _p, _p, _i, _i, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p],
     "swm_sigmoid_attention": [_p, _p, _p, _p, _p, _l, _p, _p, _i, _p, _p, _l, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p,
                               _i, _p],
@@ -93,6 +94,8 @@ def load_library() -> ctypes.CDLL:
     lib.swm_lightning_workspace_floats.argtypes = [_l, _i, _i, _i, _i, _i]
     lib.swm_masked_attention_workspace_floats.restype = _l
     lib.swm_masked_attention_workspace_floats.argtypes = [_l, _i, _i, _i, _i, _i, _i, _i, _i, _i]
+    lib.swm_gated_delta_chunked_workspace_floats.restype = _l
+    lib.swm_gated_delta_chunked_workspace_floats.argtypes = [_l, _i, _i, _i, _i]
     lib.swm_gla_workspace_floats.restype = _l
     lib.swm_gla_workspace_floats.argtypes = [_l, _i, _i, _i, _i, _i]
     if lib.swm_abi_version() != ABI_VERSION:
@@ -322,10 +325,11 @@ def causal_conv(out: torch.Tensor, x: torch.Tensor, taps: torch.Tensor, state: t
 
 def gated_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, decay_pre: torch.Tensor,
                 dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor, batch, heads: int, kv_heads: int,
-                dim: int, vdim: int) -> None:
+                dim: int, vdim: int, chunked: Optional[bool] = None) -> None:
     """The delta rule with ONE decay per head: decay_pre, beta_pre [rows, heads] (2-D views in the activation dtype),
     dt_bias, a_log fp32 [heads]; qkv fp32 [rows, 2 * kv_heads * dim + heads * vdim] from the short convolution;
-    state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim]."""
+    state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim].  ``chunked``: chunks of 32 tokens on the matrix
+    cores instead of token by token (default: when some sequence brings at least 32 tokens)."""
     _dev(out, qkv, beta_pre, decay_pre, dt_bias, a_log, state)
     for t, what in ((out, "out"), (qkv, "qkv"), (dt_bias, "dt_bias"), (a_log, "a_log"), (state, "state")):
         _f32c(t, what)
@@ -336,6 +340,19 @@ def gated_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, de
           and decay_pre.dtype == beta_pre.dtype and dt_bias.numel() == heads and a_log.numel() == heads
           and state.shape[1:] == (heads, dim, vdim) and batch.max_state_slot < state.shape[0],
           "gated_delta: shapes")
+    if chunked is None:
+        chunked = int(getattr(batch, "max_query_len", 0) or 0) >= 32
+    if chunked:
+        with _on_device_of(qkv):
+            lib = load_library()
+            need = lib.swm_gated_delta_chunked_workspace_floats(rows, n, heads, dim, vdim)
+            work = torch.empty(need, dtype=torch.float32, device=qkv.device)
+            _check(lib.swm_gated_delta_chunked(
+                out.data_ptr(), qkv.data_ptr(), beta_pre.data_ptr(), _rows(beta_pre, "beta_pre"), decay_pre.data_ptr(),
+                _rows(decay_pre, "decay_pre"), dt_bias.data_ptr(), a_log.data_ptr(), state.data_ptr(),
+                batch.q_start.data_ptr(), batch.ctx_len.data_ptr(), batch.state_slot.data_ptr(), rows, n, heads,
+                kv_heads, dim, vdim, work.data_ptr(), _act(decay_pre), _stream(qkv)))
+        return
     work = torch.empty(rows * heads * (3 * (-(-dim // 4) * 4) + 1), dtype=torch.float32, device=qkv.device)
     with _on_device_of(qkv):
         _check(load_library().swm_gated_delta(
