@@ -317,7 +317,7 @@ int swm_gated_delta(float* out, const float* qkv, const void* beta_pre, int64_t 
 
 /* The same rule in chunks of 32 tokens on the matrix cores, for steps that bring long runs (any step is right, steps of
  * few tokens per sequence are faster with swm_gated_delta): a prologue parallel over (chunk, head), then one walk over
- * each sequence's chunks.  `workspace`: swm_gated_delta_chunked_workspace_floats() floats. */
+ * each sequence's chunks.  Key sizes up to 224.  `workspace`: swm_gated_delta_chunked_workspace_floats() floats. */
 int64_t swm_gated_delta_chunked_workspace_floats(int64_t rows, int num_seqs, int heads, int dim, int vdim);
 int swm_gated_delta_chunked(float* out, const float* qkv, const void* beta_pre, int64_t beta_stride,
                             const void* decay_pre, int64_t decay_stride, const float* dt_bias, const float* a_log,

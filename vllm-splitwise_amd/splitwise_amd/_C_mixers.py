@@ -329,7 +329,7 @@ def gated_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, de
     """The delta rule with ONE decay per head: decay_pre, beta_pre [rows, heads] (2-D views in the activation dtype),
     dt_bias, a_log fp32 [heads]; qkv fp32 [rows, 2 * kv_heads * dim + heads * vdim] from the short convolution;
     state fp32 [slots, heads, dim, vdim]; out fp32 [rows, heads * vdim].  ``chunked``: chunks of 32 tokens on the matrix
-    cores instead of token by token (default: when some sequence brings at least 32 tokens)."""
+    cores instead of token by token (default: when some sequence brings at least 32 tokens; key sizes up to 224)."""
     _dev(out, qkv, beta_pre, decay_pre, dt_bias, a_log, state)
     for t, what in ((out, "out"), (qkv, "qkv"), (dt_bias, "dt_bias"), (a_log, "a_log"), (state, "state")):
         _f32c(t, what)
@@ -342,7 +342,7 @@ def gated_delta(out: torch.Tensor, qkv: torch.Tensor, beta_pre: torch.Tensor, de
           "gated_delta: shapes")
     if chunked is None:
         chunked = int(getattr(batch, "max_query_len", 0) or 0) >= 32
-    if chunked:
+    if chunked and dim <= 224:                                 # larger keys: the chunks' operands outgrow the LDS
         with _on_device_of(qkv):
             lib = load_library()
             need = lib.swm_gated_delta_chunked_workspace_floats(rows, n, heads, dim, vdim)
