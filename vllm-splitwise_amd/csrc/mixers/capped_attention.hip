@@ -2,7 +2,9 @@
 // scores (cap * tanh(score / cap)), an optional mask (a sliding window, or chunks counted from position 0 inside which
 // a position sees the earlier ones), an optional extra term exp(0) in the softmax's denominator (a key of score 0
 // that carries no value) and an optional sigmoid gate on the output.  A cache slot's keys and values are addressed
-// by strides, so values may be a part of the key rows (attention over a latent shared by all heads).
+// by strides, so values may be a part of the key rows (attention over a latent shared by all heads).  Given a bias per
+// query head the same kernels run WITHOUT a softmax: a seen key weighs sigmoid(score + bias), nothing is normalised over
+// the keys, and parts are joined by plain addition.
 // Scores, softmax weights and the weighted sum of values are fp32: both products run on the matrix cores in
 // fp32 (v_mfma_f32_32x32x2_f32), keys and values are widened when they come from a bf16 cache.
 //
